@@ -1,0 +1,135 @@
+/*
+ * teletron_op.h — C ABI of the MI355X (gfx950) fused normalisation kernels.
+ *
+ * This is the drop-in boundary for TeleTron's `teletron_op` native ops.  Every
+ * entry point takes plain device pointers, sizes and a HIP stream handle; no
+ * torch types appear in any signature.  All tensors are row-major and
+ * contiguous: `rows x cols` bf16 for activations, bf16 for parameters, fp32 for
+ * per-row statistics and for parameter gradients.
+ *
+ * Two groups of entry points:
+ *
+ *  1. The native contract (tt_adaln_*, tt_rmsnorm_*): backward consumes the
+ *     forward *input* x and recomputes the row statistics, so nothing but x has
+ *     to be saved; parameter gradients are fp32 and may be per-sample
+ *     ([n_batches, cols], n_batches = rows / rows_per_batch).
+ *  2. The reference-compatible contract (tt_launch_*): argument for argument the
+ *     launchers that the reference's pybind glue calls, including the saved
+ *     x_norm / y tensors and bf16 parameter gradients.
+ *
+ * Return value: 0 (TT_OK) on success, otherwise one of the TT_ERR_* codes;
+ * tt_error_string() maps a code to text and tt_last_hip_error() returns the
+ * hipError_t recorded by the calling thread's last TT_ERR_HIP.  Kernels are
+ * enqueued on `stream` (NULL = the default stream) of the *current* device and
+ * the calls do not synchronise.  The library keeps no mutable global state, so
+ * calls from several host threads on different streams are safe.
+ */
+#ifndef TELETRON_OP_H_
+#define TELETRON_OP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define TT_API __attribute__((visibility("default")))
+#else
+#define TT_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TT_OK 0
+#define TT_ERR_INVALID_ARGUMENT 1  /* null pointer, non-positive size, rows % rows_per_batch != 0 */
+#define TT_ERR_UNSUPPORTED 2       /* shape outside what the kernels cover (cols > TT_MAX_COLS) */
+#define TT_ERR_WORKSPACE 3         /* workspace pointer null or smaller than *_workspace_bytes() */
+#define TT_ERR_HIP 4               /* a HIP runtime call or kernel launch failed */
+
+#define TT_MAX_COLS 32768
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+TT_API int tt_version(void);
+TT_API const char* tt_error_string(int code);
+TT_API int tt_last_hip_error(void);
+
+/* ------------------------------------------------------------------ fused AdaLN
+ * y = LayerNorm_noaffine(x) * (1 + scale) + shift
+ *
+ * Replaces launch_adaln_forward (teletron_op/fused_adaln/include/adaln_kernel.h:21-30,
+ * teletron_op/fused_adaln/adaln_forward.cu:198-220) for any `cols`, with
+ * per-sample modulation: scale/shift are [n_batches, cols] bf16 where row r uses
+ * batch r / rows_per_batch (pass rows_per_batch = rows for a single [cols] vector,
+ * the reference's only mode, adaln_forward.cu:171-172).  Unlike the reference it
+ * does not emit x_norm; `mean` and `rstd` ([rows] fp32) are optional (NULL to skip).
+ */
+TT_API int tt_adaln_forward(void* y, const void* x, const void* scale, const void* shift,
+                     float* mean, float* rstd,
+                     int64_t rows, int64_t cols, int64_t rows_per_batch,
+                     float eps, void* stream);
+
+/* Backward of the above.  Replaces launch_adaln_backward + launch_adaln_scale_shift_backward
+ * (adaln_kernel.h:32-46, adaln_backward.cu:129-151, scale_shift_backward.cu:129-147):
+ *   g = dy * (1 + scale);  dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat))
+ *   dscale[b, c] = sum_{rows of batch b} dy * x_hat;  dshift[b, c] = sum dy
+ * Inputs dy, x: [rows, cols] bf16; scale: [n_batches, cols] bf16.
+ * Outputs dx: [rows, cols] bf16; dscale, dshift: [n_batches, cols] fp32.
+ * `workspace` holds the per-workgroup partial column sums; it must be at least
+ * tt_adaln_backward_workspace_bytes() and 16-byte aligned.  The result is
+ * bitwise reproducible run to run (fixed summation order, no atomics).
+ */
+TT_API int tt_adaln_backward(void* dx, float* dscale, float* dshift,
+                      const void* dy, const void* x, const void* scale,
+                      void* workspace, size_t workspace_bytes,
+                      int64_t rows, int64_t cols, int64_t rows_per_batch,
+                      float eps, void* stream);
+TT_API size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch);
+
+/* ------------------------------------------------------------------ fused RMSNorm
+ * y = x * rsqrt(mean(x^2) + eps) * weight
+ *
+ * Replaces launch_rms_forward (teletron_op/fused_rmsnorm/include/rmsnorm_kernel.h:5-12,
+ * teletron_op/fused_rmsnorm/rms_forward.cu:102-121) for any `cols` (the reference
+ * covers cols == 128 only).  `rstd` ([rows] fp32) is optional.
+ */
+TT_API int tt_rmsnorm_forward(void* y, const void* x, const void* weight, float* rstd,
+                       int64_t rows, int64_t cols, float eps, void* stream);
+
+/* Backward: replaces launch_rms_backward + launch_rms_weight_backward
+ * (rmsnorm_kernel.h:14-25, rms_backward.cu:91-112, weight_backward.cu:212-260):
+ *   g = dy * weight;  dx = rstd * (g - x_hat * mean(g * x_hat));  dweight[c] = sum_rows dy * x_hat
+ * Consumes x (not the forward output) and never divides by weight.
+ * dweight: [cols] fp32.  Workspace as for tt_adaln_backward.
+ */
+TT_API int tt_rmsnorm_backward(void* dx, float* dweight,
+                        const void* dy, const void* x, const void* weight,
+                        void* workspace, size_t workspace_bytes,
+                        int64_t rows, int64_t cols, float eps, void* stream);
+TT_API size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
+
+/* ------------------------------------------------------------------ two-step backward
+ * The backward entry points above are these two steps back to back.  They are
+ * exported so that a caller can time the streaming kernel on its own, or sum the
+ * per-workgroup partials of several devices before the final reduction.
+ * (No counterpart in the reference, whose column reductions are separate kernels
+ * that re-read dout and x_norm: scale_shift_backward.cu:49-126, weight_backward.cu:59-145.)
+ *
+ * Step 1 writes dx and, into `workspace`, partial column sums laid out as
+ * [n_batches][*n_partials][n_acc][cols] fp32 with n_acc = 2 (dscale, dshift) for
+ * AdaLN and 1 for RMSNorm.  Step 2 reduces over the n_partials axis in a fixed order.
+ */
+TT_API int tt_adaln_backward_partials(void* dx, const void* dy, const void* x, const void* scale,
+                               void* workspace, size_t workspace_bytes, int* n_partials,
+                               int64_t rows, int64_t cols, int64_t rows_per_batch,
+                               float eps, void* stream);
+TT_API int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x, const void* weight,
+                                 void* workspace, size_t workspace_bytes, int* n_partials,
+                                 int64_t rows, int64_t cols, float eps, void* stream);
+/* out0 / out1: [n_batches, cols] fp32; out1 is NULL when n_acc == 1. */
+TT_API int tt_reduce_partials(float* out0, float* out1, const void* workspace,
+                       int n_batches, int n_partials, int n_acc, int64_t cols, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TELETRON_OP_H_ */

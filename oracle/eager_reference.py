@@ -1,0 +1,60 @@
+"""PyTorch-eager restatement of the model-side ops the fused kernels replace.
+TEST INFRASTRUCTURE / CPU BASELINE ONLY: never imported by the shipped package.
+
+These are the ops TeleTron runs when ``FUSED_KERNELS`` is off
+(``teletron_op/README.md:6``), written out again here so they can be timed on the
+host CPU next to the GPU kernels and compared with the float64 oracle:
+
+* ``EagerRMSNorm``  follows ``teletron/models/wan/wan_model.py:113-124``:
+  ``norm(x.float()).to(x.dtype) * weight`` (note the cast back to bf16 *before*
+  the multiply by ``weight``).
+* ``EagerAdaLN``    follows ``wan_model.py:222-223,236`` / ``:271-278``:
+  ``nn.LayerNorm(dim, eps, elementwise_affine=False)`` then
+  ``modulate(x, shift, scale) = x * (1 + scale) + shift`` (``wan_model.py:77-78``).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+
+class EagerRMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        xf = x.float()
+        normed = xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return normed.to(x.dtype) * self.weight
+
+
+class EagerAdaLN(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.norm = nn.LayerNorm(dim, eps=eps, elementwise_affine=False)
+
+    def forward(self, x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+        return self.norm(x) * (1 + scale) + shift
+
+
+def eager_rmsnorm_fwd_bwd(x, gamma, dy, eps):
+    """One forward + autograd backward; returns (y, dx, dgamma)."""
+    mod = EagerRMSNorm(x.shape[-1], eps)
+    mod.weight = nn.Parameter(gamma.detach().clone())
+    xr = x.detach().clone().requires_grad_(True)
+    y = mod(xr)
+    y.backward(dy)
+    return y.detach(), xr.grad, mod.weight.grad
+
+
+def eager_adaln_fwd_bwd(x, scale, shift, dy, eps):
+    """One forward + autograd backward; returns (y, dx, dscale, dshift)."""
+    mod = EagerAdaLN(x.shape[-1], eps)
+    xr = x.detach().clone().requires_grad_(True)
+    sc = scale.detach().clone().requires_grad_(True)
+    sh = shift.detach().clone().requires_grad_(True)
+    y = mod(xr, sh, sc)
+    y.backward(dy)
+    return y.detach(), xr.grad, sc.grad, sh.grad

@@ -1,0 +1,178 @@
+"""CPU oracle for the fused AdaLN / RMSNorm path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in float64 on the CPU, the arithmetic that TeleTron's
+``teletron_op`` fused normalisation kernels stand for.  Only the test-suite,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import it; the shipped package never does (its ops raise when the HIP library
+is missing instead of falling back to anything on the CPU).
+
+Semantic sources in the reference (all paths relative to the reference root):
+
+* RMSNorm:   ``teletron/models/wan/wan_model.py:113-124``
+             (``x * rsqrt(mean(x^2, -1) + eps)`` then ``* weight``) and the fused
+             kernel ``teletron_op/fused_rmsnorm/rms_forward.cu:63-98``.
+* AdaLN:     ``nn.LayerNorm(dim, eps, elementwise_affine=False)`` followed by
+             ``modulate`` = ``x * (1 + scale) + shift``
+             (``teletron/models/wan/wan_model.py:77-78,222-223,236,241``) and the
+             fused kernel ``teletron_op/fused_adaln/adaln_forward.cu:156-193``.
+* AdaLN bwd: ``teletron_op/fused_adaln/adaln_backward.cu:85-125`` (dx) and
+             ``scale_shift_backward.cu:84-92`` (dshift = sum_rows dy,
+             dscale = sum_rows dy * x_hat); per-sample ``[B,1,C]`` reductions as in
+             ``teletron/core/context_parallel/layers.py:46-53``.
+* RMSNorm bwd: ``teletron_op/fused_rmsnorm/rms_backward.cu:64-87`` (dx) and
+             ``weight_backward.cu:84-103`` (dweight = sum_rows dy * x_hat).
+
+The reference kernels chain several bf16 roundings; the parity contract for this
+build is the *formula evaluated without intermediate rounding*, which is what is
+written here.  Every function below is pinned in ``tests/test_oracle.py`` against
+torch's library routines (``F.layer_norm`` / ``F.rms_norm`` + autograd), against
+central finite differences of a pure-Python scalar implementation, and against
+closed-form special cases.  No function here is "parity unpinned".
+
+Shapes: ``x``, ``dy`` are ``[B, S, C]`` (any leading dims are flattened by the
+callers); ``scale`` / ``shift`` are ``[B, C]`` (or ``[1, C]`` broadcast over B);
+``gamma`` is ``[C]``.  All inputs are converted to float64.
+"""
+from __future__ import annotations
+
+import torch
+
+F64 = torch.float64
+
+
+def _f64(t: torch.Tensor) -> torch.Tensor:
+    return t.detach().to(device="cpu", dtype=F64)
+
+
+def _bsc(x: torch.Tensor, n_batches: int) -> torch.Tensor:
+    c = x.shape[-1]
+    return _f64(x).reshape(n_batches, -1, c)
+
+
+def _param(p: torch.Tensor, n_batches: int, c: int) -> torch.Tensor:
+    p = _f64(p).reshape(-1, c)
+    if p.shape[0] == 1 and n_batches > 1:
+        p = p.expand(n_batches, c)
+    assert p.shape[0] == n_batches, (p.shape, n_batches)
+    return p
+
+
+# --------------------------------------------------------------------------- AdaLN
+def adaln_stats(x: torch.Tensor, eps: float, n_batches: int = 1):
+    """Row mean and 1/sqrt(biased variance + eps) (adaln_forward.cu:156-165)."""
+    xb = _bsc(x, n_batches)
+    mean = xb.mean(dim=-1, keepdim=True)
+    var = ((xb - mean) ** 2).mean(dim=-1, keepdim=True)
+    rstd = 1.0 / torch.sqrt(var + eps)
+    return mean, rstd
+
+
+def adaln_forward(x, scale, shift, eps: float, n_batches: int = 1):
+    """y = LayerNorm_noaffine(x) * (1 + scale) + shift.
+
+    Returns ``(y, x_hat, mean, rstd)``; ``y`` / ``x_hat`` have x's shape,
+    ``mean`` / ``rstd`` have one entry per row.
+    """
+    c = x.shape[-1]
+    xb = _bsc(x, n_batches)
+    sc = _param(scale, n_batches, c)[:, None, :]
+    sh = _param(shift, n_batches, c)[:, None, :]
+    mean, rstd = adaln_stats(x, eps, n_batches)
+    x_hat = (xb - mean) * rstd
+    y = x_hat * (1.0 + sc) + sh
+    return (y.reshape(x.shape), x_hat.reshape(x.shape),
+            mean.reshape(-1), rstd.reshape(-1))
+
+
+def adaln_backward(dy, x, scale, eps: float, n_batches: int = 1):
+    """Gradients of ``adaln_forward`` w.r.t. x, scale, shift.
+
+    dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat)),  g = dy * (1 + scale)
+    dscale[b, c] = sum_s dy * x_hat ;  dshift[b, c] = sum_s dy.
+    Returns ``(dx, dscale[B,C], dshift[B,C])``.
+    """
+    c = x.shape[-1]
+    xb = _bsc(x, n_batches)
+    dyb = _bsc(dy, n_batches)
+    sc = _param(scale, n_batches, c)[:, None, :]
+    mean, rstd = adaln_stats(x, eps, n_batches)
+    x_hat = (xb - mean) * rstd
+    g = dyb * (1.0 + sc)
+    m1 = g.mean(dim=-1, keepdim=True)
+    m2 = (g * x_hat).mean(dim=-1, keepdim=True)
+    dx = rstd * (g - m1 - x_hat * m2)
+    dscale = (dyb * x_hat).sum(dim=1)
+    dshift = dyb.sum(dim=1)
+    return dx.reshape(x.shape), dscale, dshift
+
+
+# --------------------------------------------------------------------------- RMSNorm
+def rmsnorm_stats(x: torch.Tensor, eps: float):
+    """1/sqrt(mean(x^2) + eps) per row (rms_forward.cu:71-81, wan_model.py:119-120)."""
+    xf = _f64(x)
+    ms = (xf * xf).mean(dim=-1, keepdim=True)
+    return 1.0 / torch.sqrt(ms + eps)
+
+
+def rmsnorm_forward(x, gamma, eps: float):
+    """y = x * rsqrt(mean(x^2) + eps) * gamma.  Returns ``(y, x_hat, rstd)``."""
+    xf = _f64(x)
+    rstd = rmsnorm_stats(x, eps)
+    x_hat = xf * rstd
+    y = x_hat * _f64(gamma)
+    return y, x_hat, rstd.reshape(-1)
+
+
+def rmsnorm_backward(dy, x, gamma, eps: float):
+    """Gradients of ``rmsnorm_forward`` w.r.t. x and gamma.
+
+    dx = rstd * (g - x_hat * mean(g * x_hat)),  g = dy * gamma
+    dgamma[c] = sum_rows dy * x_hat.
+    Returns ``(dx, dgamma[C])``.
+    """
+    c = x.shape[-1]
+    xf = _f64(x)
+    dyf = _f64(dy)
+    rstd = rmsnorm_stats(x, eps)
+    x_hat = xf * rstd
+    g = dyf * _f64(gamma)
+    m2 = (g * x_hat).mean(dim=-1, keepdim=True)
+    dx = rstd * (g - x_hat * m2)
+    dgamma = (dyf * x_hat).reshape(-1, c).sum(dim=0)
+    return dx, dgamma
+
+
+# --------------------------------------------------------------------------- chunked variants
+def adaln_backward_param_grads_chunked(dy, x, eps: float, n_batches: int = 1, chunk_rows: int = 4096):
+    """dscale / dshift only, streamed over row chunks so that full-size shapes
+    (hundreds of millions of elements) never materialise float64 copies."""
+    c = x.shape[-1]
+    xb = x.reshape(n_batches, -1, c)
+    dyb = dy.reshape(n_batches, -1, c)
+    s = xb.shape[1]
+    dscale = torch.zeros(n_batches, c, dtype=F64)
+    dshift = torch.zeros(n_batches, c, dtype=F64)
+    for b in range(n_batches):
+        for r0 in range(0, s, chunk_rows):
+            xs = _f64(xb[b, r0:r0 + chunk_rows])
+            ds = _f64(dyb[b, r0:r0 + chunk_rows])
+            mean = xs.mean(dim=-1, keepdim=True)
+            var = ((xs - mean) ** 2).mean(dim=-1, keepdim=True)
+            x_hat = (xs - mean) / torch.sqrt(var + eps)
+            dscale[b] += (ds * x_hat).sum(dim=0)
+            dshift[b] += ds.sum(dim=0)
+    return dscale, dshift
+
+
+def rmsnorm_backward_param_grads_chunked(dy, x, eps: float, chunk_rows: int = 4096):
+    """dgamma only, streamed over row chunks (see above)."""
+    c = x.shape[-1]
+    x2 = x.reshape(-1, c)
+    dy2 = dy.reshape(-1, c)
+    dgamma = torch.zeros(c, dtype=F64)
+    for r0 in range(0, x2.shape[0], chunk_rows):
+        xs = _f64(x2[r0:r0 + chunk_rows])
+        ds = _f64(dy2[r0:r0 + chunk_rows])
+        rstd = 1.0 / torch.sqrt((xs * xs).mean(dim=-1, keepdim=True) + eps)
+        dgamma += (ds * xs * rstd).sum(dim=0)
+    return dgamma

@@ -1,0 +1,85 @@
+"""Builds the HIP shared library ``libteletron_op.so`` (C ABI, no torch dependency)
+in-tree with hipcc for gfx950, and optionally the torch-facing pybind modules.
+
+Usage:  python -m teletron_amd.build [--force] [--define NAME=VALUE ...]
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+REPO_ROOT = PKG_DIR.parent
+CSRC = PKG_DIR / "csrc"
+OBJ_DIR = CSRC / "build"
+LIB_PATH = PKG_DIR / "libteletron_op.so"
+
+HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_bwd.hip", "rms_fwd.hip", "rms_bwd.hip"]
+
+# -packed-fp32-ops is switched off on purpose: the compiler must not form
+# v_pk_{add,mul,fma}_f32 from the scalar float code of these kernels.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; a ROCm toolchain is required to build teletron_amd")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(map(str, cmd)), proc.stdout, proc.stderr))
+    return proc
+
+
+def build_library(force: bool = True, defines=(), jobs: int = 8, verbose: bool = True) -> Path:
+    """Compile every HIP translation unit and link libteletron_op.so."""
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    headers = list(CSRC.glob("*.hpp")) + [REPO_ROOT / "include" / "teletron_op.h"]
+    newest_header = max(h.stat().st_mtime for h in headers)
+    dflags = ["-D" + d for d in defines]
+
+    def compile_one(name: str) -> Path:
+        src = CSRC / name
+        obj = OBJ_DIR / (Path(name).stem + ".o")
+        if (not force and obj.exists() and obj.stat().st_mtime > max(src.stat().st_mtime, newest_header)):
+            return obj
+        cmd = [hipcc(), *HIP_FLAGS, *dflags, "-I", str(REPO_ROOT / "include"), "-I", str(CSRC),
+               "-c", str(src), "-o", str(obj)]
+        if verbose:
+            print("[teletron_amd.build] hipcc", name, flush=True)
+        _run(cmd)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
+    if verbose:
+        print("[teletron_amd.build] linked", LIB_PATH, flush=True)
+    return LIB_PATH
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--force", action="store_true", help="recompile even if objects look current")
+    ap.add_argument("--define", action="append", default=[], help="extra -D for hipcc (tuning constants)")
+    ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    args = ap.parse_args(argv)
+    build_library(force=args.force or bool(args.define), defines=args.define, jobs=args.jobs)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

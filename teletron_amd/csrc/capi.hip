@@ -1,0 +1,279 @@
+// C ABI of the fused normalisation kernels: argument validation, launch planning
+// (variant, grid, workspace) and the kernel launches.  See include/teletron_op.h.
+#include "teletron_op.h"
+
+#include <atomic>
+#include <mutex>
+#include <unordered_map>
+
+#include "kernel_table.hpp"
+
+namespace tt {
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+int hip_fail(hipError_t e) {
+  g_last_hip_error = static_cast<int>(e);
+  (void)hipGetLastError();  // clear the sticky launch error, it has been recorded
+  return TT_ERR_HIP;
+}
+
+struct DeviceInfo {
+  int cus = 0;
+};
+
+int current_device_cus(int* cus) {
+  static std::mutex mu;
+  static DeviceInfo info[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e);
+  if (dev < 0 || dev >= 64) return TT_ERR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(mu);
+  if (info[dev].cus == 0) {
+    int n = 0;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return hip_fail(e);
+    info[dev].cus = n > 0 ? n : 1;
+  }
+  *cus = info[dev].cus;
+  return TT_OK;
+}
+
+// Resident workgroups per CU for a kernel, from the HIP occupancy calculator (cached).
+int resident_wgs_per_cu(const KernelInfo& k, int* out) {
+  static std::mutex mu;
+  static std::unordered_map<const void*, int> cache;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = cache.find(k.fn);
+    if (it != cache.end()) { *out = it->second; return TT_OK; }
+  }
+  int n = 0;
+  hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k.fn, k.threads, 0);
+  if (e != hipSuccess) return hip_fail(e);
+  if (n < 1) n = 1;
+  std::lock_guard<std::mutex> lock(mu);
+  cache[k.fn] = n;
+  *out = n;
+  return TT_OK;
+}
+
+std::atomic<int> g_wgs_per_cu_override{0};
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+struct Plan {
+  KernelInfo k;
+  int64_t n_batches = 0;
+  int64_t n_tiles = 0;   // per batch
+  int grid_x = 0;        // workgroups per batch == partial sums per batch
+  int packs = 0;
+};
+
+enum Dir { kFwd, kBwd };
+
+// Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
+constexpr int kMaxWgsPerCu = 8;
+
+int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan) {
+  if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0)
+    return TT_ERR_INVALID_ARGUMENT;
+  if (cols > TT_MAX_COLS) return TT_ERR_UNSUPPORTED;
+  if (cols % kPack != 0) return TT_ERR_UNSUPPORTED;
+  const int packs = static_cast<int>(cols / kPack);
+  const bool narrow = packs <= kNarrowMaxPacks;
+  const int idx = narrow ? select_narrow(packs) : select_wide(packs);
+  if (idx < 0) return TT_ERR_UNSUPPORTED;
+  const int slots = narrow ? kNarrowL[idx] : 64 * kWideW[idx] * kWideP[idx];
+  const bool full = (slots == packs);
+  KernelInfo k;
+  if (kind == kAdaLN) k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full) : adaln_bwd_kernel(narrow, idx, full);
+  else                k = dir == kFwd ? rms_fwd_kernel(narrow, idx, full) : rms_bwd_kernel(narrow, idx, full);
+  if (!k.fn) return TT_ERR_UNSUPPORTED;
+
+  int cus = 0, per_cu = 0;
+  int rc = current_device_cus(&cus);
+  if (rc != TT_OK) return rc;
+  rc = resident_wgs_per_cu(k, &per_cu);
+  if (rc != TT_OK) return rc;
+  const int ov = g_wgs_per_cu_override.load(std::memory_order_relaxed);
+  if (ov > 0) per_cu = ov;
+  if (per_cu > kMaxWgsPerCu) per_cu = kMaxWgsPerCu;
+
+  plan->k = k;
+  plan->packs = packs;
+  plan->n_batches = rows / rows_per_batch;
+  plan->n_tiles = (rows_per_batch + k.tile_rows - 1) / k.tile_rows;
+  if (plan->n_batches > 65535) return TT_ERR_UNSUPPORTED;
+  int64_t gx = (int64_t)per_cu * cus / plan->n_batches;
+  if (gx < 1) gx = 1;
+  if (gx > plan->n_tiles) gx = plan->n_tiles;
+  plan->grid_x = static_cast<int>(gx);
+  return TT_OK;
+}
+
+size_t partial_bytes(const Plan& p, int n_acc, int64_t cols) {
+  return (size_t)p.n_batches * p.grid_x * n_acc * cols * sizeof(float);
+}
+
+// Workspace bound that does not depend on the launch-time occupancy query.
+size_t workspace_bound(int n_acc, int64_t rows, int64_t cols, int64_t rows_per_batch) {
+  if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0) return 0;
+  int cus = 0;
+  if (current_device_cus(&cus) != TT_OK) cus = 256;
+  const int64_t n_batches = rows / rows_per_batch;
+  int64_t gx = (int64_t)kMaxWgsPerCu * cus / n_batches;
+  if (gx < 1) gx = 1;
+  if (gx > rows_per_batch) gx = rows_per_batch;
+  return (size_t)n_batches * gx * n_acc * cols * sizeof(float);
+}
+
+template <typename Args>
+int launch(const Plan& p, Args& args, void* stream) {
+  void* kargs[] = {&args};
+  hipError_t e = hipLaunchKernel(p.k.fn, dim3(p.grid_x, (unsigned)p.n_batches, 1), dim3(p.k.threads, 1, 1),
+                                 kargs, 0, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e);
+  return TT_OK;
+}
+
+int forward(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd,
+            int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!y || !x || !p0 || (kind == kAdaLN && !p1)) return TT_ERR_INVALID_ARGUMENT;
+  if (!aligned16(y) || !aligned16(x) || !aligned16(p0) || !aligned16(p1)) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p);
+  if (rc != TT_OK) return rc;
+  FwdArgs a;
+  a.y = y; a.x = x; a.p0 = p0; a.p1 = p1; a.mean = mean; a.rstd = rstd;
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
+  a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
+  return launch(p, a, stream);
+}
+
+int backward_partials(int kind, void* dx, const void* dy, const void* x, const void* p0,
+                      void* workspace, size_t workspace_bytes, int* n_partials,
+                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  if (n_partials) *n_partials = 0;
+  if (rows == 0) return TT_OK;
+  if (!dx || !dy || !x || !p0) return TT_ERR_INVALID_ARGUMENT;
+  if (!aligned16(dx) || !aligned16(dy) || !aligned16(x) || !aligned16(p0)) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kind, kBwd, rows, cols, rows_per_batch, &p);
+  if (rc != TT_OK) return rc;
+  const int n_acc = kind == kAdaLN ? 2 : 1;
+  if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;
+  BwdArgs a;
+  a.dx = dx; a.dy = dy; a.x = x; a.p0 = p0; a.partials = static_cast<float*>(workspace);
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
+  a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
+  rc = launch(p, a, stream);
+  if (rc == TT_OK && n_partials) *n_partials = p.grid_x;
+  return rc;
+}
+
+int reduce(float* out0, float* out1, const void* workspace, int n_batches, int n_partials, int n_acc,
+           int64_t cols, void* stream) {
+  if (n_batches == 0) return TT_OK;
+  if (!out0 || !workspace || n_batches < 0 || n_batches > 65535 || n_partials <= 0 || cols <= 0 ||
+      cols > TT_MAX_COLS || (n_acc != 1 && n_acc != 2) || (n_acc == 2 && !out1))
+    return TT_ERR_INVALID_ARGUMENT;
+  const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)n_batches, 1);
+  const float* ws = static_cast<const float*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (n_acc == 2) hipLaunchKernelGGL(reduce_partials<2>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols);
+  else            hipLaunchKernelGGL(reduce_partials<1>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e);
+  return TT_OK;
+}
+
+}  // namespace
+}  // namespace tt
+
+using namespace tt;
+
+extern "C" {
+
+int tt_version(void) { return 100; }
+
+const char* tt_error_string(int code) {
+  switch (code) {
+    case TT_OK: return "ok";
+    case TT_ERR_INVALID_ARGUMENT: return "invalid argument (null pointer, non-positive size, or rows not a multiple of rows_per_batch)";
+    case TT_ERR_UNSUPPORTED: return "unsupported shape or alignment";
+    case TT_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case TT_ERR_HIP: return "HIP runtime error (see tt_last_hip_error)";
+    default: return "unknown error code";
+  }
+}
+
+int tt_last_hip_error(void) { return g_last_hip_error; }
+
+// Tuning hook (not part of the public header): force the number of resident
+// workgroups per CU that launch plans assume; 0 restores the occupancy query.
+TT_API void tt_debug_set_wgs_per_cu(int n) { g_wgs_per_cu_override.store(n < 0 ? 0 : n); }
+
+int tt_adaln_forward(void* y, const void* x, const void* scale, const void* shift, float* mean, float* rstd,
+                     int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  return forward(kAdaLN, y, x, scale, shift, mean, rstd, rows, cols, rows_per_batch, eps, stream);
+}
+
+int tt_rmsnorm_forward(void* y, const void* x, const void* weight, float* rstd,
+                       int64_t rows, int64_t cols, float eps, void* stream) {
+  return forward(kRMS, y, x, weight, nullptr, nullptr, rstd, rows, cols, rows, eps, stream);
+}
+
+size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch) {
+  return workspace_bound(2, rows, cols, rows_per_batch);
+}
+size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
+  return workspace_bound(1, rows, cols, rows);
+}
+
+int tt_adaln_backward_partials(void* dx, const void* dy, const void* x, const void* scale,
+                               void* workspace, size_t workspace_bytes, int* n_partials,
+                               int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  return backward_partials(kAdaLN, dx, dy, x, scale, workspace, workspace_bytes, n_partials,
+                           rows, cols, rows_per_batch, eps, stream);
+}
+int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x, const void* weight,
+                                 void* workspace, size_t workspace_bytes, int* n_partials,
+                                 int64_t rows, int64_t cols, float eps, void* stream) {
+  return backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, n_partials,
+                           rows, cols, rows, eps, stream);
+}
+
+int tt_reduce_partials(float* out0, float* out1, const void* workspace,
+                       int n_batches, int n_partials, int n_acc, int64_t cols, void* stream) {
+  return reduce(out0, out1, workspace, n_batches, n_partials, n_acc, cols, stream);
+}
+
+int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, const void* x, const void* scale,
+                      void* workspace, size_t workspace_bytes,
+                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dscale || !dshift) return TT_ERR_INVALID_ARGUMENT;
+  int n_partials = 0;
+  int rc = backward_partials(kAdaLN, dx, dy, x, scale, workspace, workspace_bytes, &n_partials,
+                             rows, cols, rows_per_batch, eps, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dscale, dshift, workspace, (int)(rows / rows_per_batch), n_partials, 2, cols, stream);
+}
+
+int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
+                        void* workspace, size_t workspace_bytes,
+                        int64_t rows, int64_t cols, float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dweight) return TT_ERR_INVALID_ARGUMENT;
+  int n_partials = 0;
+  int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
+                             rows, cols, rows, eps, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, stream);
+}
+
+}  // extern "C"

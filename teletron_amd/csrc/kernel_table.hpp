@@ -1,0 +1,139 @@
+// Table of compiled kernel variants and the host-side lookup that maps a row
+// width to one of them.  Each of the four kernel families (AdaLN / RMSNorm x
+// forward / backward) is instantiated in its own translation unit through the
+// lookup templates below, so the families compile in parallel.
+#pragma once
+#include "norm_kernels.hpp"
+
+namespace tt {
+
+struct KernelInfo {
+  const void* fn;   // __global__ function taking one FwdArgs / BwdArgs by value
+  int threads;      // workgroup size
+  int tile_rows;    // rows one workgroup consumes per loop iteration
+};
+
+// Wide variants: (index, W waves per row, P packs per lane).  A row of `packs`
+// 128-bit packs runs on the variant with the fewest lane slots 64*W*P >= packs.
+#define TT_WIDE_LIST(X) \
+  X(0, 1, 1) X(1, 2, 1) X(2, 3, 1) X(3, 4, 1) X(4, 3, 2) X(5, 4, 2) X(6, 5, 2) \
+  X(7, 6, 2) X(8, 8, 2) X(9, 12, 2) X(10, 16, 2) X(11, 16, 4)
+constexpr int kNumWide = 12;
+constexpr int kWideW[kNumWide] = {1, 2, 3, 4, 3, 4, 5, 6, 8, 12, 16, 16};
+constexpr int kWideP[kNumWide] = {1, 1, 1, 1, 2, 2, 2, 2, 2, 2, 2, 4};
+
+// Narrow variants: (index, L lanes per row).
+#define TT_NARROW_LIST(X) X(0, 1) X(1, 2) X(2, 4) X(3, 8) X(4, 16) X(5, 32)
+constexpr int kNumNarrow = 6;
+constexpr int kNarrowL[kNumNarrow] = {1, 2, 4, 8, 16, 32};
+constexpr int kNarrowMaxPacks = 32;
+constexpr int kMaxPacks = 64 * 16 * 4;
+
+// ---- tuning constants (rows in flight per row group, row groups per workgroup)
+#ifndef TT_FWD_R
+#define TT_FWD_R 2
+#endif
+#ifndef TT_FWD_Q
+#define TT_FWD_Q 1
+#endif
+#ifndef TT_BWD_R
+#define TT_BWD_R 1
+#endif
+#ifndef TT_BWD_Q
+#define TT_BWD_Q 1
+#endif
+#ifndef TT_NARROW_FWD_R
+#define TT_NARROW_FWD_R 4
+#endif
+#ifndef TT_NARROW_BWD_R
+#define TT_NARROW_BWD_R 2
+#endif
+#ifndef TT_NARROW_NW
+#define TT_NARROW_NW 4
+#endif
+
+constexpr int clampQ(int q, int W) { return (q * W > 16) ? (16 / W > 0 ? 16 / W : 1) : q; }
+constexpr int fwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_FWD_R; }
+constexpr int fwd_wide_Q(int W, int P) { return clampQ(TT_FWD_Q, W); }
+constexpr int bwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_BWD_R; }
+constexpr int bwd_wide_Q(int W, int P) { return clampQ(TT_BWD_Q, W); }
+
+// Index of the wide variant for `packs` (> kNarrowMaxPacks), or -1.
+inline int select_wide(int packs) {
+  int best = -1, best_slots = 1 << 30;
+  for (int i = 0; i < kNumWide; ++i) {
+    const int slots = 64 * kWideW[i] * kWideP[i];
+    // fewest slots wins; on a tie the later entry (more packs per lane, fewer waves) wins
+    if (slots >= packs && slots <= best_slots) { best = i; best_slots = slots; }
+  }
+  return best;
+}
+inline int select_narrow(int packs) {
+  for (int i = 0; i < kNumNarrow; ++i)
+    if (kNarrowL[i] >= packs) return i;
+  return -1;
+}
+
+template <int KIND, int W, int P, bool FULL>
+KernelInfo info_fwd_wide() {
+  constexpr int R = fwd_wide_R(W, P), Q = fwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_fwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R};
+}
+template <int KIND, int W, int P, bool FULL>
+KernelInfo info_bwd_wide() {
+  constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_bwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R};
+}
+template <int KIND, int L, bool FULL>
+KernelInfo info_fwd_narrow() {
+  constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&norm_fwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L)};
+}
+template <int KIND, int L, bool FULL>
+KernelInfo info_bwd_narrow() {
+  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L)};
+}
+
+template <int KIND>
+KernelInfo lookup_fwd(bool narrow, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L) case i: return full ? info_fwd_narrow<KIND, L, true>() : info_fwd_narrow<KIND, L, false>();
+      TT_NARROW_LIST(X)
+#undef X
+    }
+  } else {
+    switch (idx) {
+#define X(i, W, P) case i: return full ? info_fwd_wide<KIND, W, P, true>() : info_fwd_wide<KIND, W, P, false>();
+      TT_WIDE_LIST(X)
+#undef X
+    }
+  }
+  return {nullptr, 0, 0};
+}
+template <int KIND>
+KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L) case i: return full ? info_bwd_narrow<KIND, L, true>() : info_bwd_narrow<KIND, L, false>();
+      TT_NARROW_LIST(X)
+#undef X
+    }
+  } else {
+    switch (idx) {
+#define X(i, W, P) case i: return full ? info_bwd_wide<KIND, W, P, true>() : info_bwd_wide<KIND, W, P, false>();
+      TT_WIDE_LIST(X)
+#undef X
+    }
+  }
+  return {nullptr, 0, 0};
+}
+
+// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, rms_fwd.hip, rms_bwd.hip).
+KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
+KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
+KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
+KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
+
+}  // namespace tt

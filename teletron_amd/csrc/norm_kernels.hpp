@@ -1,0 +1,611 @@
+// Streaming kernels for fused AdaLN / RMSNorm, forward and backward, on gfx950.
+//
+// Two shapes of kernel cover every row width that is a multiple of 8:
+//
+//  * "wide"   (more than 32 packs per row): a row is owned by a *row group* of
+//    W waves; lane l of wave w owns the packs  p*64*W + w*64 + l  (p < P), so
+//    each load instruction of a wave is one contiguous 1 KiB segment.  A
+//    workgroup holds Q row groups and walks the rows of one batch in tiles of
+//    Q*R rows.  The row stays in registers between the statistics pass and the
+//    output pass, so x (and dy) are read from HBM exactly once.
+//  * "narrow" (at most 32 packs per row): L = 2^k lanes own one row, a wave
+//    carries 64/L rows per load and the row reductions never leave the wave.
+//
+// Column ownership is fixed for the lifetime of a workgroup.  The parameters a
+// lane needs therefore live in registers as fp32, and in backward the lane's
+// share of dscale/dshift/dgamma is accumulated in fp32 registers over all rows
+// the workgroup visits, then written once as a per-workgroup partial.  A second
+// kernel (reduce_partials) sums the partials in a fixed order: no atomics, so
+// the parameter gradients are bitwise reproducible.
+#pragma once
+#include "common.hpp"
+
+namespace tt {
+
+enum Kind : int { kAdaLN = 0, kRMS = 1 };
+
+struct FwdArgs {
+  void* y;
+  const void* x;
+  const void* p0;   // AdaLN: scale [B, C];  RMSNorm: weight [C]
+  const void* p1;   // AdaLN: shift [B, C];  RMSNorm: unused
+  float* mean;      // optional [rows]
+  float* rstd;      // optional [rows]
+  int64_t rows_per_batch;
+  int64_t n_tiles;  // tiles per batch
+  int cols;
+  int packs;        // cols / 8
+  float eps;
+  float inv_cols;
+};
+
+struct BwdArgs {
+  void* dx;
+  const void* dy;
+  const void* x;
+  const void* p0;    // AdaLN: scale [B, C];  RMSNorm: weight [C]
+  float* partials;   // [B][gridDim.x][NACC][C]
+  int64_t rows_per_batch;
+  int64_t n_tiles;
+  int cols;
+  int packs;
+  float eps;
+  float inv_cols;
+};
+
+// Sum NV values over the W waves of one row group.  `buf` points at W*NV floats
+// of LDS private to (reduction phase parity, row group).  Callers alternate two
+// buffers between consecutive reductions, which makes one barrier per reduction
+// sufficient: a wave can only overwrite a buffer after passing the barrier of
+// the reduction in between, which every wave reaches after its reads.
+template <int W, int NV>
+__device__ __forceinline__ void rowgroup_allsum(float (&v)[NV], float* buf, int w, int lane) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = wave_allsum(v[i]);
+  if constexpr (W > 1) {
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) buf[w * NV + i] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      float t = buf[i];
+#pragma unroll
+      for (int ww = 1; ww < W; ++ww) t += buf[ww * NV + i];
+      v[i] = t;
+    }
+  }
+}
+
+// ============================================================================ wide forward
+template <int KIND, int W, int P, int R, int Q, bool FULL>
+__global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  __shared__ float red[2][Q][W * R];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = wave / W;
+  const int w = wave - q * W;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+
+  int col[P];
+  bool act[P];
+  float g[P][8], sh[P][8];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int pk = p * 64 * W + w * 64 + lane;
+    act[p] = FULL || pk < a.packs;
+    col[p] = pk * kPack;
+    u32x4 r0 = {0, 0, 0, 0}, r1 = {0, 0, 0, 0};
+    if (act[p]) {
+      r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col[p]);
+      if constexpr (ADALN) r1 = load_cached(a.p1, b * C + col[p]);
+    }
+    unpack8(r0, g[p]);
+    unpack8(r1, sh[p]);
+    if constexpr (ADALN) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) g[p][j] += 1.0f;
+    }
+  }
+
+  unsigned phase = 0;
+  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t row0 = tile * (Q * R) + q * R;
+    float xf[R][P][8];
+    bool rv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      rv[r] = row0 + r < S;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        u32x4 raw = {0, 0, 0, 0};
+        if (rv[r] && act[p]) raw = load_stream(a.x, (size_t)((b * S + row0 + r) * C + col[p]));
+        unpack8(raw, xf[r][p]);
+      }
+    }
+
+    float mean[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) mean[r] = 0.f;
+    if constexpr (ADALN) {
+      float s[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float t = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) t += xf[r][p][j];
+        s[r] = t;
+      }
+      rowgroup_allsum<W, R>(s, red[phase & 1][q], w, lane);
+      ++phase;
+#pragma unroll
+      for (int r = 0; r < R; ++r) mean[r] = s[r] * a.inv_cols;
+    }
+
+    float v[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float t = 0.f;
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float d = xf[r][p][j];
+          if constexpr (ADALN) {
+            d -= mean[r];
+            if constexpr (!FULL) d = act[p] ? d : 0.f;
+            xf[r][p][j] = d;
+          }
+          t = fmaf(d, d, t);
+        }
+      v[r] = t;
+    }
+    rowgroup_allsum<W, R>(v, red[phase & 1][q], w, lane);
+    ++phase;
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float rstd = rsqrtf(v[r] * a.inv_cols + a.eps);
+      if (rv[r]) {
+        const int64_t row = b * S + row0 + r;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          if (act[p]) {
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float xh = xf[r][p][j] * rstd;
+              o[j] = ADALN ? fmaf(xh, g[p][j], sh[p][j]) : xh * g[p][j];
+            }
+            store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
+          }
+        }
+        if (w == 0 && lane == 0) {
+          if (ADALN && a.mean) a.mean[row] = mean[r];
+          if (a.rstd) a.rstd[row] = rstd;
+        }
+      }
+    }
+  }
+}
+
+// ============================================================================ wide backward
+template <int KIND, int W, int P, int R, int Q, bool FULL>
+__global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  constexpr int NACC = ADALN ? 2 : 1;
+  constexpr int NV = ADALN ? 3 : 2;  // reduced values per row in the main phase
+  __shared__ float red[2][Q][W * R * NV];
+  __shared__ __attribute__((aligned(16))) float comb[Q > 1 ? 64 * W * P * 8 : 4];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = wave / W;
+  const int w = wave - q * W;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+
+  int col[P];
+  bool act[P];
+  float g[P][8];
+  float acc0[P][8];  // dscale / dgamma
+  float acc1[P][8];  // dshift (AdaLN only)
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int pk = p * 64 * W + w * 64 + lane;
+    act[p] = FULL || pk < a.packs;
+    col[p] = pk * kPack;
+    u32x4 r0 = {0, 0, 0, 0};
+    if (act[p]) r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col[p]);
+    unpack8(r0, g[p]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (ADALN) g[p][j] += 1.0f;
+      acc0[p][j] = 0.f;
+      acc1[p][j] = 0.f;
+    }
+  }
+
+  unsigned phase = 0;
+  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t row0 = tile * (Q * R) + q * R;
+    float xf[R][P][8], df[R][P][8];
+    bool rv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      rv[r] = row0 + r < S;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        u32x4 rx = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
+        if (rv[r] && act[p]) {
+          const size_t off = (size_t)((b * S + row0 + r) * C + col[p]);
+          rx = load_stream(a.x, off);
+          rd = load_stream(a.dy, off);
+        }
+        unpack8(rx, xf[r][p]);
+        unpack8(rd, df[r][p]);
+      }
+    }
+
+    float mean[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) mean[r] = 0.f;
+    if constexpr (ADALN) {
+      float s[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float t = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) t += xf[r][p][j];
+        s[r] = t;
+      }
+      rowgroup_allsum<W, R>(s, red[phase & 1][q], w, lane);
+      ++phase;
+#pragma unroll
+      for (int r = 0; r < R; ++r) mean[r] = s[r] * a.inv_cols;
+    }
+
+    // One pass gives sum d^2, sum g*d and (AdaLN) sum g, with d = x - mean and g = dy * param.
+    float red_v[R * NV];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float sv = 0.f, sh_ = 0.f, sg = 0.f;
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float d = xf[r][p][j];
+          if constexpr (ADALN) {
+            d -= mean[r];
+            if constexpr (!FULL) d = act[p] ? d : 0.f;
+            xf[r][p][j] = d;
+          }
+          const float gg = df[r][p][j] * g[p][j];
+          sv = fmaf(d, d, sv);
+          sh_ = fmaf(gg, d, sh_);
+          if constexpr (ADALN) sg += gg;
+        }
+      red_v[r * NV + 0] = sv;
+      red_v[r * NV + 1] = sh_;
+      if constexpr (ADALN) red_v[r * NV + 2] = sg;
+    }
+    rowgroup_allsum<W, R * NV>(red_v, red[phase & 1][q], w, lane);
+    ++phase;
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float rstd = rsqrtf(red_v[r * NV + 0] * a.inv_cols + a.eps);
+      // dx = rstd*g - rstd*mean(g) - x_hat * rstd*mean(g*x_hat),  mean(g*x_hat) = rstd * sum(g*d) / C
+      const float k2 = -(rstd * rstd) * (red_v[r * NV + 1] * a.inv_cols);
+      const float k1 = ADALN ? -rstd * (red_v[r * NV + 2] * a.inv_cols) : 0.f;
+      const int64_t row = b * S + row0 + r;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float xh = xf[r][p][j] * rstd;
+          const float dyv = df[r][p][j];
+          acc0[p][j] = fmaf(dyv, xh, acc0[p][j]);
+          if constexpr (ADALN) acc1[p][j] += dyv;
+          o[j] = fmaf(xh, k2, fmaf(dyv * g[p][j], rstd, k1));
+        }
+        if (rv[r] && act[p]) store_stream(a.dx, (size_t)(row * C + col[p]), pack8(o));
+      }
+    }
+  }
+
+  // Fold the Q row groups of this workgroup into group 0, in group order.
+  if constexpr (Q > 1) {
+#pragma unroll
+    for (int acc = 0; acc < NACC; ++acc) {
+      for (int qq = 1; qq < Q; ++qq) {
+        __syncthreads();
+        if (q == qq) {
+#pragma unroll
+          for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              comb[((p * W + w) * 64 + lane) * 8 + j] = acc == 0 ? acc0[p][j] : acc1[p][j];
+        }
+        __syncthreads();
+        if (q == 0) {
+#pragma unroll
+          for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float t = comb[((p * W + w) * 64 + lane) * 8 + j];
+              if (acc == 0) acc0[p][j] += t; else acc1[p][j] += t;
+            }
+        }
+      }
+    }
+  }
+
+  if (q == 0) {
+    float* base = a.partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      if (act[p]) {
+        f32x4* d0 = reinterpret_cast<f32x4*>(base + col[p]);
+        d0[0] = f32x4{acc0[p][0], acc0[p][1], acc0[p][2], acc0[p][3]};
+        d0[1] = f32x4{acc0[p][4], acc0[p][5], acc0[p][6], acc0[p][7]};
+        if constexpr (ADALN) {
+          f32x4* d1 = reinterpret_cast<f32x4*>(base + C + col[p]);
+          d1[0] = f32x4{acc1[p][0], acc1[p][1], acc1[p][2], acc1[p][3]};
+          d1[1] = f32x4{acc1[p][4], acc1[p][5], acc1[p][6], acc1[p][7]};
+        }
+      }
+    }
+  }
+}
+
+// ============================================================================ narrow forward
+// L lanes per row (one pack each), 64/L rows per wave per load, R loads in flight,
+// NW independent waves per workgroup.  A tile is NW*R*(64/L) consecutive rows.
+template <int KIND, int L, int R, int NW, bool FULL>
+__global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  constexpr int RPW = 64 / L;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int pi = lane & (L - 1);
+  const int ri = lane / L;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+  const bool act = FULL || pi < a.packs;
+  const int col = pi * kPack;
+
+  float g[8], sh[8];
+  {
+    u32x4 r0 = {0, 0, 0, 0}, r1 = {0, 0, 0, 0};
+    if (act) {
+      r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col);
+      if constexpr (ADALN) r1 = load_cached(a.p1, b * C + col);
+    }
+    unpack8(r0, g);
+    unpack8(r1, sh);
+    if constexpr (ADALN) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) g[j] += 1.0f;
+    }
+  }
+
+  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+    float xf[R][8];
+    bool rv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t rr = rbase + r * RPW;
+      rv[r] = rr < S;
+      u32x4 raw = {0, 0, 0, 0};
+      if (rv[r] && act) raw = load_stream(a.x, (size_t)((b * S + rr) * C + col));
+      unpack8(raw, xf[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float mean = 0.f;
+      if constexpr (ADALN) {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t += xf[r][j];
+        mean = group_allsum<L>(t) * a.inv_cols;
+      }
+      float v = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float d = xf[r][j];
+        if constexpr (ADALN) {
+          d -= mean;
+          if constexpr (!FULL) d = act ? d : 0.f;
+          xf[r][j] = d;
+        }
+        v = fmaf(d, d, v);
+      }
+      v = group_allsum<L>(v);
+      const float rstd = rsqrtf(v * a.inv_cols + a.eps);
+      if (rv[r] && act) {
+        const int64_t row = b * S + rbase + r * RPW;
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float xh = xf[r][j] * rstd;
+          o[j] = ADALN ? fmaf(xh, g[j], sh[j]) : xh * g[j];
+        }
+        store_stream(a.y, (size_t)(row * C + col), pack8(o));
+        if (pi == 0) {
+          if (ADALN && a.mean) a.mean[row] = mean;
+          if (a.rstd) a.rstd[row] = rstd;
+        }
+      }
+    }
+  }
+}
+
+// ============================================================================ narrow backward
+template <int KIND, int L, int R, int NW, bool FULL>
+__global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  constexpr int NACC = ADALN ? 2 : 1;
+  constexpr int RPW = 64 / L;
+  __shared__ __attribute__((aligned(16))) float comb[NW][NACC][L * 8];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int pi = lane & (L - 1);
+  const int ri = lane / L;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+  const bool act = FULL || pi < a.packs;
+  const int col = pi * kPack;
+
+  float g[8], acc0[8], acc1[8];
+  {
+    u32x4 r0 = {0, 0, 0, 0};
+    if (act) r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col);
+    unpack8(r0, g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (ADALN) g[j] += 1.0f;
+      acc0[j] = 0.f;
+      acc1[j] = 0.f;
+    }
+  }
+
+  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+    float xf[R][8], df[R][8];
+    bool rv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t rr = rbase + r * RPW;
+      rv[r] = rr < S;
+      u32x4 rx = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
+      if (rv[r] && act) {
+        const size_t off = (size_t)((b * S + rr) * C + col);
+        rx = load_stream(a.x, off);
+        rd = load_stream(a.dy, off);
+      }
+      unpack8(rx, xf[r]);
+      unpack8(rd, df[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float mean = 0.f;
+      if constexpr (ADALN) {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t += xf[r][j];
+        mean = group_allsum<L>(t) * a.inv_cols;
+      }
+      float sv = 0.f, sh_ = 0.f, sg = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float d = xf[r][j];
+        if constexpr (ADALN) {
+          d -= mean;
+          if constexpr (!FULL) d = act ? d : 0.f;
+          xf[r][j] = d;
+        }
+        const float gg = df[r][j] * g[j];
+        sv = fmaf(d, d, sv);
+        sh_ = fmaf(gg, d, sh_);
+        if constexpr (ADALN) sg += gg;
+      }
+      sv = group_allsum<L>(sv);
+      sh_ = group_allsum<L>(sh_);
+      if constexpr (ADALN) sg = group_allsum<L>(sg);
+      const float rstd = rsqrtf(sv * a.inv_cols + a.eps);
+      const float k2 = -(rstd * rstd) * (sh_ * a.inv_cols);
+      const float k1 = ADALN ? -rstd * (sg * a.inv_cols) : 0.f;
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float xh = xf[r][j] * rstd;
+        const float dyv = df[r][j];
+        acc0[j] = fmaf(dyv, xh, acc0[j]);
+        if constexpr (ADALN) acc1[j] += dyv;
+        o[j] = fmaf(xh, k2, fmaf(dyv * g[j], rstd, k1));
+      }
+      if (rv[r] && act) store_stream(a.dx, (size_t)((b * S + rbase + r * RPW) * C + col), pack8(o));
+    }
+  }
+
+  // Fold the 64/L row slots of the wave (lanes with equal pi), then the waves.
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+#pragma unroll
+    for (int m = L; m < 64; m <<= 1) {
+      acc0[j] += __shfl_xor(acc0[j], m, 64);
+      if constexpr (ADALN) acc1[j] += __shfl_xor(acc1[j], m, 64);
+    }
+  }
+  if (ri == 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      comb[wave][0][pi * 8 + j] = acc0[j];
+      if constexpr (ADALN) comb[wave][NACC - 1][pi * 8 + j] = acc1[j];
+    }
+  }
+  __syncthreads();
+  float* base = a.partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
+  for (int i = threadIdx.x; i < NACC * L * 8; i += 64 * NW) {
+    const int acc = i / (L * 8);
+    const int c = i - acc * (L * 8);
+    if (c < C) {
+      float t = comb[0][acc][c];
+#pragma unroll
+      for (int ww = 1; ww < NW; ++ww) t += comb[ww][acc][c];
+      base[(size_t)acc * C + c] = t;
+    }
+  }
+}
+
+// ============================================================================ second pass
+// out[acc][b][c] = sum_j partials[b][j][acc][c], j in a fixed order: 16 waves take
+// the partials j = wave, wave+16, ... and are then folded in wave order through LDS.
+template <int NACC>
+__global__ __launch_bounds__(1024) void reduce_partials(float* __restrict__ out0, float* __restrict__ out1,
+                                                        const float* __restrict__ partials,
+                                                        int n_partials, int cols) {
+  __shared__ float fold[16][NACC][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int64_t b = blockIdx.y;
+  float s[NACC];
+#pragma unroll
+  for (int acc = 0; acc < NACC; ++acc) s[acc] = 0.f;
+  if (c < cols) {
+    const float* base = partials + (size_t)b * n_partials * NACC * cols + c;
+    for (int j = wave; j < n_partials; j += 16) {
+#pragma unroll
+      for (int acc = 0; acc < NACC; ++acc) s[acc] += base[((size_t)j * NACC + acc) * cols];
+    }
+  }
+#pragma unroll
+  for (int acc = 0; acc < NACC; ++acc) fold[wave][acc][lane] = s[acc];
+  __syncthreads();
+  if (wave < NACC && c < cols) {
+    float t = fold[0][wave][lane];
+#pragma unroll
+    for (int ww = 1; ww < 16; ++ww) t += fold[ww][wave][lane];
+    float* out = wave == 0 ? out0 : out1;
+    out[(size_t)b * cols + c] = t;
+  }
+}
+
+}  // namespace tt

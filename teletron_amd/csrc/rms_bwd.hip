@@ -1,0 +1,6 @@
+// Instantiates the rms bwd kernel family (one translation unit per family so they build in parallel).
+#include "kernel_table.hpp"
+
+namespace tt {
+KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full) { return lookup_bwd<kRMS>(narrow, idx, full); }
+}  // namespace tt

@@ -1,0 +1,115 @@
+"""``torch.autograd.Function`` / ``nn.Module`` surface of the fused ops.
+
+``AdaLNModelFunction`` and ``RMSNormModelFunction`` keep the call signatures and
+return orders documented for TeleTron's ops (``teletron_op/README.md:20-92`` and
+``:104-172``): ``apply(x, scale, shift, epsilon, cols)`` / ``apply(x, weight,
+epsilon, cols)``, backward returning ``(dx, dscale, dshift, None, None)`` /
+``(dx, dweight, None, None)``.  Differences, all widening:
+
+* any ``cols`` that is a multiple of 8 (the reference: 3072 / 128 only);
+* ``scale`` / ``shift`` may be per-sample ``[B, 1, C]`` as produced by
+  ``(modulation + t_mod).chunk(...)`` in ``teletron/models/wan/wan_model.py:234-235``;
+* backward saves ``x`` (not ``x_norm`` / the forward output) and recomputes the
+  row statistics; parameter gradients are reduced in fp32 and cast once to the
+  parameter's dtype.
+
+``FusedRMSNorm`` has the constructor and ``weight`` state-dict key of the Wan
+``RMSNorm`` (``wan_model.py:113-124``); ``FusedAdaLN`` replaces
+``modulate(nn.LayerNorm(dim, eps, elementwise_affine=False)(x), shift, scale)``
+(``wan_model.py:77-78,222-223,236``).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+from torch.autograd import Function
+
+from . import ops
+
+
+class AdaLNModelFunction(Function):
+    @staticmethod
+    def forward(ctx, x, scale, shift, epsilon, cols):
+        if x.numel() % cols != 0 or x.shape[-1] != cols:
+            raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols}")
+        ctx.eps = float(epsilon)
+        ctx.scale_meta = (scale.shape, scale.dtype)
+        ctx.shift_meta = (shift.shape, shift.dtype)
+        x = x.contiguous()
+        scale_c = scale.detach().to(torch.bfloat16).contiguous()
+        y = ops.adaln_forward(x, scale_c, shift.detach(), ctx.eps)
+        ctx.save_for_backward(x, scale_c)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, scale_c = ctx.saved_tensors
+        dx, dscale, dshift = ops.adaln_backward(grad_output.contiguous(), x, scale_c, ctx.eps)
+        (sc_shape, sc_dtype), (sh_shape, sh_dtype) = ctx.scale_meta, ctx.shift_meta
+        dx = dx if ctx.needs_input_grad[0] else None
+        dscale = dscale.to(sc_dtype).reshape(sc_shape) if ctx.needs_input_grad[1] else None
+        dshift = dshift.to(sh_dtype).reshape(sh_shape) if ctx.needs_input_grad[2] else None
+        return dx, dscale, dshift, None, None
+
+
+class RMSNormModelFunction(Function):
+    @staticmethod
+    def forward(ctx, x, weight, epsilon, cols):
+        if x.numel() % cols != 0 or x.shape[-1] != cols:
+            raise ValueError(f"Input size {x.numel()} not divisible by cols {cols}")
+        ctx.eps = float(epsilon)
+        ctx.weight_meta = (weight.shape, weight.dtype)
+        x = x.contiguous()
+        weight_c = weight.detach().to(torch.bfloat16).contiguous()
+        y = ops.rmsnorm_forward(x, weight_c, ctx.eps)
+        ctx.save_for_backward(x, weight_c)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight_c = ctx.saved_tensors
+        dx, dweight = ops.rmsnorm_backward(grad_output.contiguous(), x, weight_c, ctx.eps)
+        w_shape, w_dtype = ctx.weight_meta
+        dx = dx if ctx.needs_input_grad[0] else None
+        dweight = dweight.to(w_dtype).reshape(w_shape) if ctx.needs_input_grad[1] else None
+        return dx, dweight, None, None
+
+
+def fused_adaln(x, shift, scale, eps: float = 1e-6):
+    """``modulate(layer_norm(x), shift, scale)`` in one kernel (argument order of ``modulate``)."""
+    return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
+
+
+def fused_rmsnorm(x, weight, eps: float = 1e-5):
+    return RMSNormModelFunction.apply(x, weight, eps, x.shape[-1])
+
+
+class FusedRMSNorm(nn.Module):
+    """Drop-in for the Wan ``RMSNorm(dim, eps)`` module: same constructor, same ``weight`` key."""
+
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.dim = dim
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return RMSNormModelFunction.apply(x, self.weight, self.eps, self.dim)
+
+    def extra_repr(self) -> str:
+        return f"{self.dim}, eps={self.eps}"
+
+
+class FusedAdaLN(nn.Module):
+    """LayerNorm without affine parameters fused with ``x * (1 + scale) + shift``; parameter-free."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.dim = dim
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+        return AdaLNModelFunction.apply(x, scale, shift, self.eps, self.dim)
+
+    def extra_repr(self) -> str:
+        return f"{self.dim}, eps={self.eps}"

@@ -1,0 +1,142 @@
+"""Tensor-level front end of the C ABI: validation, output allocation, stream and
+device handling.  Every function launches HIP kernels through ``libteletron_op.so``
+on the current stream of the input's device; nothing here computes on the CPU.
+
+Shapes: ``x`` / ``dy`` are bf16 with the normalised dimension last.  AdaLN
+``scale`` / ``shift`` hold ``n_batches * cols`` elements (``[C]``, ``[1,1,C]``,
+``[B,1,C]`` ...): the flattened rows of ``x`` are split into ``n_batches`` equal
+consecutive groups, group ``b`` using modulation vector ``b``.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import cabi
+
+BF16 = torch.bfloat16
+
+
+def _require(cond: bool, exc, msg: str):
+    if not cond:
+        raise exc(msg)
+
+
+def _check_act(name: str, t: torch.Tensor, cols: int) -> torch.Tensor:
+    _require(isinstance(t, torch.Tensor), TypeError, f"{name} must be a torch.Tensor")
+    _require(t.is_cuda, ValueError, f"{name} must live on a GPU (got device {t.device}); there is no CPU path")
+    _require(t.dtype == BF16, TypeError, f"{name} must be bfloat16 (got {t.dtype})")
+    _require(cols > 0 and t.numel() % cols == 0, ValueError,
+             f"Input tensor size {t.numel()} not divisible by cols {cols}")
+    _require(t.dim() >= 1 and t.shape[-1] == cols, ValueError,
+             f"{name}: last dimension {tuple(t.shape)} must equal cols {cols}")
+    return t.contiguous()
+
+
+def _check_param(name: str, p: torch.Tensor, ref: torch.Tensor, cols: int) -> torch.Tensor:
+    _require(isinstance(p, torch.Tensor), TypeError, f"{name} must be a torch.Tensor")
+    _require(p.device == ref.device, ValueError, f"{name} is on {p.device}, input on {ref.device}")
+    _require(p.dim() >= 1 and p.shape[-1] == cols, ValueError,
+             f"{name}: last dimension of {tuple(p.shape)} must equal cols {cols}")
+    if p.dtype != BF16:
+        p = p.to(BF16)
+    return p.contiguous()
+
+
+def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int, int]:
+    rows = x.numel() // cols
+    nb = scale.numel() // cols
+    _require(nb >= 1 and (rows == 0 or rows % nb == 0), ValueError,
+             f"scale/shift hold {nb} vectors, which does not divide the {rows} rows of the input")
+    return rows, nb, (rows // nb if nb else rows)
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def adaln_forward(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float,
+                  return_stats: bool = False):
+    """y = LayerNorm_noaffine(x) * (1 + scale) + shift.  Returns y, or (y, mean, rstd)."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    scale = _check_param("scale", scale, x, cols)
+    shift = _check_param("shift", shift, x, cols)
+    _require(scale.numel() == shift.numel(), ValueError, "scale and shift must have the same number of elements")
+    rows, nb, rpb = _batches(x, scale, cols)
+    y = torch.empty_like(x)
+    mean = rstd = None
+    if return_stats:
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    if rows:
+        with torch.cuda.device(x.device):
+            cabi.call("tt_adaln_forward", y.data_ptr(), x.data_ptr(), scale.data_ptr(), shift.data_ptr(),
+                      _ptr(mean), _ptr(rstd), rows, cols, rpb, float(eps), _stream(x))
+    return (y, mean, rstd) if return_stats else y
+
+
+def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: float):
+    """Returns (dx bf16 like x, dscale fp32 [n_batches, C], dshift fp32 [n_batches, C])."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    dy = _check_act("dy", dy, cols)
+    _require(dy.numel() == x.numel() and dy.device == x.device, ValueError, "dy must match x in size and device")
+    scale = _check_param("scale", scale, x, cols)
+    rows, nb, rpb = _batches(x, scale, cols)
+    dx = torch.empty_like(x)
+    if rows == 0:
+        z = torch.zeros(nb, cols, dtype=torch.float32, device=x.device)
+        return dx, z, z.clone()
+    dscale = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
+    dshift = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        ws_bytes = cabi.load().tt_adaln_backward_workspace_bytes(rows, cols, rpb)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        cabi.call("tt_adaln_backward", dx.data_ptr(), dscale.data_ptr(), dshift.data_ptr(),
+                  dy.data_ptr(), x.data_ptr(), scale.data_ptr(), ws.data_ptr(), ws_bytes,
+                  rows, cols, rpb, float(eps), _stream(x))
+    return dx, dscale, dshift
+
+
+def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, return_stats: bool = False):
+    """y = x * rsqrt(mean(x^2) + eps) * weight.  Returns y, or (y, rstd)."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    weight = _check_param("weight", weight, x, cols)
+    _require(weight.numel() == cols, ValueError, f"weight must have {cols} elements, got {weight.numel()}")
+    rows = x.numel() // cols
+    y = torch.empty_like(x)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device) if return_stats else None
+    if rows:
+        with torch.cuda.device(x.device):
+            cabi.call("tt_rmsnorm_forward", y.data_ptr(), x.data_ptr(), weight.data_ptr(), _ptr(rstd),
+                      rows, cols, float(eps), _stream(x))
+    return (y, rstd) if return_stats else y
+
+
+def rmsnorm_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """Returns (dx bf16 like x, dweight fp32 [C])."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    dy = _check_act("dy", dy, cols)
+    _require(dy.numel() == x.numel() and dy.device == x.device, ValueError, "dy must match x in size and device")
+    weight = _check_param("weight", weight, x, cols)
+    _require(weight.numel() == cols, ValueError, f"weight must have {cols} elements, got {weight.numel()}")
+    rows = x.numel() // cols
+    dx = torch.empty_like(x)
+    if rows == 0:
+        return dx, torch.zeros(cols, dtype=torch.float32, device=x.device)
+    dweight = torch.empty(cols, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        ws_bytes = cabi.load().tt_rmsnorm_backward_workspace_bytes(rows, cols)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        cabi.call("tt_rmsnorm_backward", dx.data_ptr(), dweight.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                  weight.data_ptr(), ws.data_ptr(), ws_bytes, rows, cols, float(eps), _stream(x))
+    return dx, dweight

@@ -1,0 +1,82 @@
+"""Seeded synthetic inputs for the benchmark / parity configurations.
+
+Draw order is fixed (x, then the parameters, then dy) from one ``torch.Generator``
+so that the same seed regenerates the same tensors on any host.  Values are drawn
+in fp32 on the CPU and rounded to bf16.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class Workload:
+    name: str
+    op: str                      # "adaln" | "rmsnorm"
+    shape: Tuple[int, ...]       # activation shape, normalised dim last
+    param_shape: Tuple[int, ...]
+    eps: float = 1e-6
+    note: str = ""
+
+    @property
+    def cols(self) -> int:
+        return self.shape[-1]
+
+    @property
+    def rows(self) -> int:
+        n = 1
+        for d in self.shape[:-1]:
+            n *= d
+        return n
+
+    @property
+    def elements(self) -> int:
+        return self.rows * self.cols
+
+    def algorithmic_bytes(self, direction: str = "fwd+bwd") -> int:
+        """Compulsory HBM traffic: bf16 activations once in / once out, plus parameters in
+        and fp32 parameter gradients out (the partial-sum workspace is not counted)."""
+        e = self.elements
+        n_param = 1
+        for d in self.param_shape:
+            n_param *= d
+        n_vec = 2 if self.op == "adaln" else 1
+        fwd = 4 * e + n_vec * n_param * 2
+        bwd = 6 * e + n_param * 2 + n_vec * n_param * 4
+        return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
+
+
+WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
+    Workload("rmsnorm_small", "rmsnorm", (2, 4096, 1536), (1536,), note="CPU-runnable reference case"),
+    Workload("adaln_wan14b", "adaln", (1, 75600, 5120), (1, 1, 5120), note="Wan2.1-14B AdaLN, 81-frame 720P"),
+    Workload("rmsnorm_wan14b_qk", "rmsnorm", (1, 75600, 5120), (5120,), note="Wan2.1-14B QK-norm (per tensor)"),
+    Workload("rmsnorm_hunyuan_head", "rmsnorm", (1, 118800, 24, 128), (128,), note="HunyuanVideo per-head norm (per tensor)"),
+    Workload("adaln_wan1p3b_batched", "adaln", (4, 32760, 1536), (4, 1, 1536), note="per-sample modulation"),
+    Workload("adaln_odd", "adaln", (3, 5000, 1000), (3, 1, 1000), note="125 packs per row: ragged wave tail"),
+]}
+
+
+def make_inputs(w: Workload, seed: int = 0, device="cpu", rows: Optional[int] = None):
+    """Returns a dict of bf16 tensors: x, dy and scale/shift or gamma.
+
+    ``rows`` (optional) truncates the sequence dimension (dim -2 of a 3-D shape, dim 1
+    of the 4-D per-head shape) for bounded CPU samples; parameters are unaffected.
+    """
+    shape = list(w.shape)
+    if rows is not None:
+        shape[1] = rows
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    out = {}
+    if w.op == "adaln":
+        shift = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        scale = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        out["shift"], out["scale"] = shift, scale
+    else:
+        out["gamma"] = 1.0 + 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+    dy = torch.randn(shape, generator=g, dtype=torch.float32)
+    out["x"], out["dy"] = x, dy
+    return {k: v.to(torch.bfloat16).to(device) for k, v in out.items()}

@@ -1,0 +1,140 @@
+"""GPU parity at the benchmark configurations, full size, through the C ABI.
+
+Small configurations are compared element by element with the float64 oracle.  At
+the full Wan / HunyuanVideo shapes (hundreds of millions of elements) the oracle is
+applied to a sample of rows for y / dx / statistics (rows are independent), the
+parameter gradients are checked against the oracle streamed over *all* rows, and
+size-independent properties are asserted on the whole output: dx rows sum to zero
+(AdaLN), the column sums of dshift add up to the grand total of dy, and repeated
+runs are bitwise identical.  Tolerances are those stated in test_gpu_parity.py.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+from teletron_amd.workloads import WORKLOADS, make_inputs
+from test_gpu_parity import DEV, assert_bf16_close, assert_grad_close
+
+pytestmark = pytest.mark.gpu
+
+
+def sample_rows(n_rows, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.cat([torch.arange(0, min(8, n_rows)), torch.arange(max(0, n_rows - 8), n_rows),
+                     torch.randint(0, n_rows, (k,), generator=g)])
+    return torch.unique(idx)
+
+
+def test_rmsnorm_small_config_full_oracle():
+    from teletron_amd import ops
+    w = WORKLOADS["rmsnorm_small"]
+    t = make_inputs(w, seed=0)
+    x, gamma, dy = t["x"], t["gamma"], t["dy"]
+    y, rstd = ops.rmsnorm_forward(x.to(DEV), gamma.to(DEV), w.eps, return_stats=True)
+    dx, dgamma = ops.rmsnorm_backward(dy.to(DEV), x.to(DEV), gamma.to(DEV), w.eps)
+    yo, _, ro = O.rmsnorm_forward(x, gamma, w.eps)
+    dxo, dgo = O.rmsnorm_backward(dy, x, gamma, w.eps)
+    assert_bf16_close(y, yo, "y")
+    assert_bf16_close(dx, dxo, "dx")
+    torch.testing.assert_close(rstd.double().cpu(), ro, rtol=1e-5, atol=0)
+    assert_grad_close(dgamma, dgo, w.rows, "dgamma")
+
+
+def test_adaln_odd_config_full_oracle():
+    from teletron_amd import ops
+    w = WORKLOADS["adaln_odd"]
+    t = make_inputs(w, seed=0)
+    nb = w.shape[0]
+    y = ops.adaln_forward(t["x"].to(DEV), t["scale"].to(DEV), t["shift"].to(DEV), w.eps)
+    dx, dscale, dshift = ops.adaln_backward(t["dy"].to(DEV), t["x"].to(DEV), t["scale"].to(DEV), w.eps)
+    yo, _, _, _ = O.adaln_forward(t["x"], t["scale"], t["shift"], w.eps, nb)
+    dxo, dsco, dsho = O.adaln_backward(t["dy"], t["x"], t["scale"], w.eps, nb)
+    assert_bf16_close(y, yo, "y")
+    assert_bf16_close(dx, dxo, "dx")
+    assert_grad_close(dscale, dsco, w.shape[1], "dscale")
+    assert_grad_close(dshift, dsho, w.shape[1], "dshift")
+
+
+def _adaln_full_size(name, chunk_rows):
+    from teletron_amd import ops
+    w = WORKLOADS[name]
+    nb, s, c = w.shape
+    t = make_inputs(w, seed=0)
+    xd, dyd, scd, shd = (t[k].to(DEV) for k in ("x", "dy", "scale", "shift"))
+    y, mean, rstd = ops.adaln_forward(xd, scd, shd, w.eps, return_stats=True)
+    dx, dscale, dshift = ops.adaln_backward(dyd, xd, scd, w.eps)
+    torch.cuda.synchronize()
+
+    # sampled rows, per batch, against the oracle
+    for b in range(nb):
+        idx = sample_rows(s, 256, seed=b)
+        xs, dys = t["x"][b, idx], t["dy"][b, idx]
+        yo, _, mo, ro = O.adaln_forward(xs, t["scale"][b], t["shift"][b], w.eps, 1)
+        dxo, _, _ = O.adaln_backward(dys, xs, t["scale"][b], w.eps, 1)
+        assert_bf16_close(y[b, idx.to(DEV)], yo, f"y batch {b}")
+        assert_bf16_close(dx[b, idx.to(DEV)], dxo, f"dx batch {b}")
+        flat = (b * s + idx).to(DEV)
+        torch.testing.assert_close(mean[flat].double().cpu(), mo, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(rstd[flat].double().cpu(), ro, rtol=1e-5, atol=0)
+
+    # parameter gradients over all rows
+    dsco, dsho = O.adaln_backward_param_grads_chunked(t["dy"], t["x"], w.eps, nb, chunk_rows)
+    assert_grad_close(dscale, dsco, s, "dscale")
+    assert_grad_close(dshift, dsho, s, "dshift")
+
+    # properties of the whole output
+    row_sums = torch.stack([dx[b].float().sum(-1).abs().max() for b in range(nb)]).max().item()
+    assert row_sums < 0.02 * math.sqrt(c), f"dx rows should sum to ~0 (bf16 rounding noise only), got {row_sums}"
+    total_dy = sum(dyd[b].double().sum().item() for b in range(nb))
+    assert abs(dshift.double().sum().item() - total_dy) < 1e-6 * nb * s * c ** 0.5
+    dx2, dscale2, dshift2 = ops.adaln_backward(dyd, xd, scd, w.eps)
+    assert torch.equal(dx, dx2) and torch.equal(dscale, dscale2) and torch.equal(dshift, dshift2)
+
+
+def test_adaln_wan14b_full_size():
+    _adaln_full_size("adaln_wan14b", 4096)
+
+
+def test_adaln_batched_full_size():
+    _adaln_full_size("adaln_wan1p3b_batched", 8192)
+
+
+def _rmsnorm_full_size(name, chunk_rows):
+    from teletron_amd import ops
+    w = WORKLOADS[name]
+    c = w.cols
+    t = make_inputs(w, seed=0)
+    x2, dy2 = t["x"].reshape(-1, c), t["dy"].reshape(-1, c)
+    xd, dyd, gd = t["x"].to(DEV), t["dy"].to(DEV), t["gamma"].to(DEV)
+    y, rstd = ops.rmsnorm_forward(xd, gd, w.eps, return_stats=True)
+    dx, dgamma = ops.rmsnorm_backward(dyd, xd, gd, w.eps)
+    torch.cuda.synchronize()
+    assert y.shape == t["x"].shape and dx.shape == t["x"].shape
+
+    idx = sample_rows(w.rows, 1024, seed=1)
+    yo, _, ro = O.rmsnorm_forward(x2[idx], t["gamma"], w.eps)
+    dxo, _ = O.rmsnorm_backward(dy2[idx], x2[idx], t["gamma"], w.eps)
+    assert_bf16_close(y.reshape(-1, c)[idx.to(DEV)], yo, "y")
+    assert_bf16_close(dx.reshape(-1, c)[idx.to(DEV)], dxo, "dx")
+    torch.testing.assert_close(rstd[idx.to(DEV)].double().cpu(), ro, rtol=1e-5, atol=0)
+
+    dgo = O.rmsnorm_backward_param_grads_chunked(dy2, x2, w.eps, chunk_rows)
+    assert_grad_close(dgamma, dgo, w.rows, "dgamma")
+
+    # with gamma == 1 the output rows have mean square ms / (ms + eps) ~ 1: whole-tensor property
+    ones = torch.ones_like(gd)
+    y1 = ops.rmsnorm_forward(xd, ones, w.eps).reshape(-1, c)
+    ms = torch.stack([blk.float().pow(2).mean(-1).sub(1).abs().max() for blk in y1.split(1 << 18)]).max().item()
+    assert ms < 8e-3, ms
+    dx2, dgamma2 = ops.rmsnorm_backward(dyd, xd, gd, w.eps)
+    assert torch.equal(dx, dx2) and torch.equal(dgamma, dgamma2)
+
+
+def test_rmsnorm_wan14b_qk_full_size():
+    _rmsnorm_full_size("rmsnorm_wan14b_qk", 4096)
+
+
+def test_rmsnorm_hunyuan_head_full_size():
+    _rmsnorm_full_size("rmsnorm_hunyuan_head", 1 << 18)

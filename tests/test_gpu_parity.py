@@ -1,0 +1,297 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the float64 oracle.
+
+Tolerances (the contract of this build, written out here):
+  * bf16 outputs y, dx:       |got - ref| <= 1e-2 + 8e-3 * |ref|
+  * fp32 row statistics:      rtol 1e-5
+  * fp32 parameter gradients: |got - ref| <= 1e-3 * |ref| + 1e-4 * sqrt(rows reduced)
+    (a column sum over M rows of O(1) terms is a random walk of size sqrt(M); a pure
+    relative bound is ill-posed where the true sum happens to be near zero).
+"""
+import glob
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    assert torch.cuda.is_available(), "GPU tests need a GPU (run with -m gpu on the GPU box)"
+    from teletron_amd import cabi
+    cabi.load()
+
+
+def assert_bf16_close(got, ref, what):
+    got = got.detach().double().cpu().reshape(-1)
+    ref = ref.double().reshape(-1)
+    err = (got - ref).abs()
+    bound = 1e-2 + 8e-3 * ref.abs()
+    bad = err > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {ref.numel()} outside tolerance, worst excess {float((err - bound).max()):.3e}"
+
+
+def assert_grad_close(got, ref, rows_reduced, what):
+    got = got.detach().double().cpu().reshape(-1)
+    ref = ref.double().reshape(-1)
+    err = (got - ref).abs()
+    bound = 1e-3 * ref.abs() + 1e-4 * math.sqrt(rows_reduced)
+    bad = err > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {ref.numel()} outside tolerance, worst err {float(err.max()):.3e}"
+
+
+def rand_bf16(*shape, seed, scale=1.0, offset=0.0):
+    g = torch.Generator().manual_seed(seed)
+    return (offset + scale * torch.randn(*shape, generator=g)).to(torch.bfloat16)
+
+
+def run_adaln(x, scale, shift, dy, eps, nb):
+    from teletron_amd import ops
+    xd, scd, shd, dyd = (t.to(DEV) for t in (x, scale, shift, dy))
+    y, mean, rstd = ops.adaln_forward(xd, scd, shd, eps, return_stats=True)
+    dx, dscale, dshift = ops.adaln_backward(dyd, xd, scd, eps)
+    torch.cuda.synchronize()
+    return y, mean, rstd, dx, dscale, dshift
+
+
+def check_adaln(x, scale, shift, dy, eps, nb, tag):
+    y, mean, rstd, dx, dscale, dshift = run_adaln(x, scale, shift, dy, eps, nb)
+    yo, _, mo, ro = O.adaln_forward(x, scale, shift, eps, nb)
+    dxo, dsco, dsho = O.adaln_backward(dy, x, scale, eps, nb)
+    rpb = x.numel() // x.shape[-1] // nb
+    assert_bf16_close(y, yo, tag + " y")
+    assert_bf16_close(dx, dxo, tag + " dx")
+    torch.testing.assert_close(mean.double().cpu(), mo, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(rstd.double().cpu(), ro, rtol=1e-5, atol=0)
+    assert_grad_close(dscale, dsco, rpb, tag + " dscale")
+    assert_grad_close(dshift, dsho, rpb, tag + " dshift")
+
+
+def check_rmsnorm(x, gamma, dy, eps, tag):
+    from teletron_amd import ops
+    xd, gd, dyd = x.to(DEV), gamma.to(DEV), dy.to(DEV)
+    y, rstd = ops.rmsnorm_forward(xd, gd, eps, return_stats=True)
+    dx, dgamma = ops.rmsnorm_backward(dyd, xd, gd, eps)
+    torch.cuda.synchronize()
+    yo, _, ro = O.rmsnorm_forward(x, gamma, eps)
+    dxo, dgo = O.rmsnorm_backward(dy, x, gamma, eps)
+    assert_bf16_close(y, yo, tag + " y")
+    assert_bf16_close(dx, dxo, tag + " dx")
+    torch.testing.assert_close(rstd.double().cpu(), ro, rtol=1e-5, atol=0)
+    assert_grad_close(dgamma, dgo, x.numel() // x.shape[-1], tag + " dgamma")
+
+
+# ------------------------------------------------------------------ golden fixtures
+def _bf16(a):
+    return torch.from_numpy(a.copy()).view(torch.bfloat16)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=os.path.basename)
+def test_golden_fixture(path):
+    d = np.load(path)
+    eps = float(d["eps"])
+    x, dy = _bf16(d["x"]), _bf16(d["dy"])
+    if "scale" in d:
+        nb = x.shape[0]
+        y, mean, rstd, dx, dscale, dshift = run_adaln(x, _bf16(d["scale"]), _bf16(d["shift"]), dy, eps, nb)
+        assert_bf16_close(y, torch.from_numpy(d["y"]), "y")
+        assert_bf16_close(dx, torch.from_numpy(d["dx"]), "dx")
+        assert_grad_close(dscale, torch.from_numpy(d["dscale"]), x.shape[1], "dscale")
+        assert_grad_close(dshift, torch.from_numpy(d["dshift"]), x.shape[1], "dshift")
+        np.testing.assert_allclose(rstd.cpu().numpy(), d["rstd"], rtol=1e-5)
+        np.testing.assert_allclose(mean.cpu().numpy(), d["mean"], rtol=1e-5, atol=1e-5)
+    else:
+        from teletron_amd import ops
+        gamma = _bf16(d["gamma"])
+        y, rstd = ops.rmsnorm_forward(x.to(DEV), gamma.to(DEV), eps, return_stats=True)
+        dx, dgamma = ops.rmsnorm_backward(dy.to(DEV), x.to(DEV), gamma.to(DEV), eps)
+        assert_bf16_close(y, torch.from_numpy(d["y"]), "y")
+        assert_bf16_close(dx, torch.from_numpy(d["dx"]), "dx")
+        assert_grad_close(dgamma, torch.from_numpy(d["dgamma"]), x.numel() // x.shape[-1], "dgamma")
+        np.testing.assert_allclose(rstd.cpu().numpy(), d["rstd"], rtol=1e-5)
+
+
+# ------------------------------------------------------------------ shape sweep: every kernel variant, ragged tails
+WIDTHS = [8, 16, 24, 64, 128, 136, 256, 264, 512, 520, 1000, 1024, 1536, 2048, 3072, 4096, 5120,
+          6144, 8192, 12288, 16384, 32768]
+
+
+@pytest.mark.parametrize("cols", WIDTHS)
+@pytest.mark.parametrize("nb,rpb", [(1, 1), (1, 67), (3, 29)])
+def test_adaln_shapes(cols, nb, rpb):
+    seed = cols * 7 + nb * 3 + rpb
+    x = rand_bf16(nb, rpb, cols, seed=seed, offset=0.5, scale=1.5)
+    scale = rand_bf16(nb, 1, cols, seed=seed + 1, scale=0.1)
+    shift = rand_bf16(nb, 1, cols, seed=seed + 2, scale=0.1)
+    dy = rand_bf16(nb, rpb, cols, seed=seed + 3)
+    check_adaln(x, scale, shift, dy, 1e-6, nb, f"adaln[{nb},{rpb},{cols}]")
+
+
+@pytest.mark.parametrize("cols", WIDTHS)
+@pytest.mark.parametrize("rows", [1, 67, 300])
+def test_rmsnorm_shapes(cols, rows):
+    seed = cols * 11 + rows
+    x = rand_bf16(rows, cols, seed=seed, scale=2.0)
+    gamma = rand_bf16(cols, seed=seed + 1, scale=0.1, offset=1.0)
+    dy = rand_bf16(rows, cols, seed=seed + 2)
+    check_rmsnorm(x, gamma, dy, 1e-6, f"rmsnorm[{rows},{cols}]")
+
+
+def test_many_rows_narrow_and_wide():
+    # enough rows that every workgroup of the persistent grid loops several times
+    x = rand_bf16(40000, 128, seed=1, scale=1.0)
+    check_rmsnorm(x, rand_bf16(128, seed=2, scale=0.1, offset=1.0), rand_bf16(40000, 128, seed=3), 1e-6, "rms 40000x128")
+    x = rand_bf16(2, 3001, 1536, seed=4)
+    check_adaln(x, rand_bf16(2, 1, 1536, seed=5, scale=0.1), rand_bf16(2, 1, 1536, seed=6, scale=0.1),
+                rand_bf16(2, 3001, 1536, seed=7), 1e-6, 2, "adaln 2x3001x1536")
+    x = rand_bf16(1, 4099, 5120, seed=8)
+    check_adaln(x, rand_bf16(1, 1, 5120, seed=9, scale=0.1), rand_bf16(1, 1, 5120, seed=10, scale=0.1),
+                rand_bf16(1, 4099, 5120, seed=11), 1e-6, 1, "adaln 4099x5120")
+
+
+def test_large_mean_rows_keep_precision():
+    # |mean| >> std: a one-pass E[x^2] - E[x]^2 variance would lose the variance here
+    x = rand_bf16(1, 33, 1024, seed=12, offset=100.0, scale=1.0)
+    check_adaln(x, rand_bf16(1, 1, 1024, seed=13, scale=0.1), rand_bf16(1, 1, 1024, seed=14, scale=0.1),
+                rand_bf16(1, 33, 1024, seed=15), 1e-6, 1, "adaln offset 100")
+
+
+def test_constant_and_zero_rows():
+    from teletron_amd import ops
+    x = torch.zeros(5, 256, dtype=torch.bfloat16)
+    x[1] = 3.0
+    x[3] = -0.5
+    scale, shift = rand_bf16(1, 256, seed=16, scale=0.1), rand_bf16(1, 256, seed=17, scale=0.1)
+    y = ops.adaln_forward(x.to(DEV), scale.to(DEV), shift.to(DEV), 1e-6)
+    # constant rows normalise to zero: y == shift exactly, no NaN/Inf
+    assert torch.equal(y.cpu(), shift.expand(5, 256))
+    yr = ops.rmsnorm_forward(x.to(DEV), torch.ones(256, dtype=torch.bfloat16, device=DEV), 1e-6)
+    assert torch.isfinite(yr.float()).all()
+    assert torch.equal(yr[0].cpu(), torch.zeros(256, dtype=torch.bfloat16))
+    dx, dg = ops.rmsnorm_backward(torch.ones(5, 256, dtype=torch.bfloat16, device=DEV), x.to(DEV),
+                                  torch.zeros(256, dtype=torch.bfloat16, device=DEV), 1e-6)
+    # weight == 0 is legal (the reference divides by it): dx == 0, dgamma finite
+    assert torch.equal(dx.cpu(), torch.zeros(5, 256, dtype=torch.bfloat16))
+    assert torch.isfinite(dg).all()
+
+
+# ------------------------------------------------------------------ reproducibility (doubles as a race detector)
+def test_param_grads_bitwise_reproducible():
+    from teletron_amd import ops
+    x = rand_bf16(2, 5003, 1536, seed=18).to(DEV)
+    dy = rand_bf16(2, 5003, 1536, seed=19).to(DEV)
+    scale = rand_bf16(2, 1, 1536, seed=20, scale=0.1).to(DEV)
+    ref = ops.adaln_backward(dy, x, scale, 1e-6)
+    for _ in range(3):
+        got = ops.adaln_backward(dy, x, scale, 1e-6)
+        for a, b in zip(ref, got):
+            assert torch.equal(a, b)
+    x = rand_bf16(70001, 128, seed=21).to(DEV)
+    dy = rand_bf16(70001, 128, seed=22).to(DEV)
+    gamma = rand_bf16(128, seed=23, scale=0.1, offset=1.0).to(DEV)
+    ref = ops.rmsnorm_backward(dy, x, gamma, 1e-6)
+    for _ in range(3):
+        got = ops.rmsnorm_backward(dy, x, gamma, 1e-6)
+        for a, b in zip(ref, got):
+            assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------ autograd surface
+def test_autograd_functions_match_oracle():
+    from teletron_amd import AdaLNModelFunction, FusedAdaLN, FusedRMSNorm, RMSNormModelFunction
+    b, s, c = 2, 129, 1536
+    x = rand_bf16(b, s, c, seed=24)
+    dy = rand_bf16(b, s, c, seed=25)
+    # strided [B,1,C] views, as produced by (modulation + t_mod).chunk(6, dim=1)
+    tmod = rand_bf16(b, 6, c, seed=26, scale=0.1).to(DEV)
+    shift_v, scale_v = tmod.chunk(6, dim=1)[0:2]
+    assert not scale_v.is_contiguous()
+    xg = x.to(DEV).requires_grad_(True)
+    tm = tmod.clone().requires_grad_(True)
+    sh, sc = tm.chunk(6, dim=1)[0:2]
+    y = AdaLNModelFunction.apply(xg, sc, sh, 1e-6, c)
+    y.backward(dy.to(DEV))
+    yo, _, _, _ = O.adaln_forward(x, scale_v.cpu(), shift_v.cpu(), 1e-6, b)
+    dxo, dsco, dsho = O.adaln_backward(dy, x, scale_v.cpu(), 1e-6, b)
+    assert_bf16_close(y, yo, "fn y")
+    assert_bf16_close(xg.grad, dxo, "fn dx")
+    assert tm.grad.shape == tmod.shape and tm.grad.dtype == torch.bfloat16
+    # grads are rounded to bf16 for bf16 parameters: compare at bf16 resolution
+    torch.testing.assert_close(tm.grad[:, 1].double().cpu(), dsco, rtol=8e-3, atol=0.05)
+    torch.testing.assert_close(tm.grad[:, 0].double().cpu(), dsho, rtol=8e-3, atol=0.05)
+    assert torch.count_nonzero(tm.grad[:, 2:]) == 0
+
+    mod = FusedAdaLN(c, eps=1e-6)
+    y2 = mod(x.to(DEV), shift_v, scale_v)
+    assert torch.equal(y2, y.detach())
+
+    norm = FusedRMSNorm(c, eps=1e-6).to(DEV)          # fp32 weight parameter, as constructed
+    assert list(norm.state_dict().keys()) == ["weight"]
+    with torch.no_grad():
+        norm.weight.copy_(rand_bf16(c, seed=27, scale=0.1, offset=1.0).float())
+    xg = x.to(DEV).requires_grad_(True)
+    y = norm(xg)
+    y.backward(dy.to(DEV))
+    gamma = norm.weight.detach().cpu()
+    yo, _, _ = O.rmsnorm_forward(x, gamma, 1e-6)
+    dxo, dgo = O.rmsnorm_backward(dy, x, gamma, 1e-6)
+    assert_bf16_close(y, yo, "rms fn y")
+    assert_bf16_close(xg.grad, dxo, "rms fn dx")
+    assert norm.weight.grad.dtype == torch.float32
+    assert_grad_close(norm.weight.grad, dgo, b * s, "rms fn dweight")
+    y3 = RMSNormModelFunction.apply(x.to(DEV), norm.weight.detach().bfloat16(), 1e-6, c)
+    assert torch.equal(y3, y.detach())
+
+
+def test_argument_errors():
+    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction, cabi, ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        RMSNormModelFunction.apply(x, w, 1e-6, 48)             # cols does not match
+    with pytest.raises(TypeError):
+        ops.rmsnorm_forward(x.float(), w, 1e-6)                 # not bf16
+    with pytest.raises(ValueError):
+        ops.rmsnorm_forward(x.cpu(), w.cpu(), 1e-6)             # CPU tensors: no fallback
+    with pytest.raises(ValueError):
+        ops.adaln_forward(x, torch.zeros(3, 64, dtype=torch.bfloat16, device=DEV),
+                          torch.zeros(3, 64, dtype=torch.bfloat16, device=DEV), 1e-6)  # 3 does not divide 4 rows
+    with pytest.raises(cabi.TeletronOpError) as ei:
+        ops.rmsnorm_forward(torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV),
+                            torch.ones(12, dtype=torch.bfloat16, device=DEV), 1e-6)   # cols % 8 != 0
+    assert ei.value.code == cabi.TT_ERR_UNSUPPORTED
+    # empty input is a no-op
+    e = torch.zeros(0, 64, dtype=torch.bfloat16, device=DEV)
+    assert ops.rmsnorm_forward(e, w, 1e-6).shape == (0, 64)
+    dx, dw = ops.rmsnorm_backward(e, e, w, 1e-6)
+    assert dx.shape == (0, 64) and torch.count_nonzero(dw) == 0
+    # workspace too small is reported, not overrun
+    lib = cabi.load()
+    dxb = torch.empty_like(x)
+    dwb = torch.empty(64, dtype=torch.float32, device=DEV)
+    ws = torch.empty(16, dtype=torch.uint8, device=DEV)
+    rc = lib.tt_rmsnorm_backward(dxb.data_ptr(), dwb.data_ptr(), x.data_ptr(), x.data_ptr(), w.data_ptr(),
+                                 ws.data_ptr(), 16, 4, 64, 1e-6, None)
+    assert rc == cabi.TT_ERR_WORKSPACE
+    torch.cuda.synchronize()
+
+
+def test_non_default_stream():
+    from teletron_amd import ops
+    x = rand_bf16(513, 1024, seed=28).to(DEV)
+    w = rand_bf16(1024, seed=29, scale=0.1, offset=1.0).to(DEV)
+    ref = ops.rmsnorm_forward(x, w, 1e-6)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        got = ops.rmsnorm_forward(x, w, 1e-6)
+    s.synchronize()
+    assert torch.equal(ref, got)
