@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused AdaLN forward + backward at the Wan2.1-14B shape on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input already
+resident in HBM: tt_adaln_forward, then tt_adaln_backward (= the streaming
+backward kernel + the reduction of its per-workgroup partial sums), through the
+C ABI.  Two complete buffer sets alternate between steps so that nothing is served
+from the 256 MB Infinity Cache (each tensor is 774 MB).
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time per step.
+`roofline` describes the dominant kernel (the streaming backward kernel), timed
+with HIP events on the launch stream inside the timed region.  `cpu_baseline` is
+the PyTorch-eager restatement of the same ops (oracle/eager_reference.py) on the
+host cores, on a bounded row sample of the same workload.
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--workload adaln_wan14b]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+REPO_ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO_ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E peak
+METRIC = "fwd+bwd HBM GB/s and % of peak, AdaLN/RMSNorm at Wan-14B shape 75600x5120"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="adaln_wan14b")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
+    ap.add_argument("--also", default="rmsnorm_wan14b_qk", help="comma list of further workloads reported under 'also'")
+    return ap.parse_args()
+
+
+class GpuWorkload:
+    """Device buffers and C-ABI launch closures for one workload (fwd, bwd-partials, reduce)."""
+
+    def __init__(self, w, n_sets=2, seed=0):
+        import torch
+        from teletron_amd import cabi
+        self.torch, self.cabi, self.w = torch, cabi, w
+        self.lib = cabi.load()
+        dev = torch.device("cuda:0")
+        self.rows, self.cols = w.rows, w.cols
+        self.nb = w.param_shape[0] if w.op == "adaln" else 1
+        self.rpb = self.rows // self.nb
+        g = torch.Generator(device=dev).manual_seed(seed)
+        bf = torch.bfloat16
+
+        def randn(*shape, scale=1.0, offset=0.0):
+            return (offset + scale * torch.randn(*shape, generator=g, device=dev, dtype=torch.float32)).to(bf)
+
+        self.sets = []
+        for _ in range(n_sets):
+            s = {"x": randn(self.rows, self.cols), "dy": randn(self.rows, self.cols),
+                 "y": torch.empty(self.rows, self.cols, dtype=bf, device=dev),
+                 "dx": torch.empty(self.rows, self.cols, dtype=bf, device=dev)}
+            self.sets.append(s)
+        if w.op == "adaln":
+            self.p0 = randn(self.nb, self.cols, scale=0.1)                 # scale
+            self.p1 = randn(self.nb, self.cols, scale=0.1)                 # shift
+            self.n_acc = 2
+            ws_bytes = self.lib.tt_adaln_backward_workspace_bytes(self.rows, self.cols, self.rpb)
+        else:
+            self.p0 = randn(self.cols, scale=0.1, offset=1.0)              # gamma
+            self.p1 = None
+            self.n_acc = 1
+            ws_bytes = self.lib.tt_rmsnorm_backward_workspace_bytes(self.rows, self.cols)
+        self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        self.g0 = torch.empty(self.nb, self.cols, dtype=torch.float32, device=dev)
+        self.g1 = torch.empty(self.nb, self.cols, dtype=torch.float32, device=dev)
+        self.n_partials = ctypes.c_int(0)
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def fwd(self, i):
+        s = self.sets[i % len(self.sets)]
+        if self.w.op == "adaln":
+            self.cabi.call("tt_adaln_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
+                           self.p1.data_ptr(), None, None, self.rows, self.cols, self.rpb, self.w.eps, self.stream)
+        else:
+            self.cabi.call("tt_rmsnorm_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(), None,
+                           self.rows, self.cols, self.w.eps, self.stream)
+
+    def bwd_partials(self, i):
+        s = self.sets[i % len(self.sets)]
+        if self.w.op == "adaln":
+            self.cabi.call("tt_adaln_backward_partials", s["dx"].data_ptr(), s["dy"].data_ptr(), s["x"].data_ptr(),
+                           self.p0.data_ptr(), self.ws.data_ptr(), self.ws.numel(), ctypes.byref(self.n_partials),
+                           self.rows, self.cols, self.rpb, self.w.eps, self.stream)
+        else:
+            self.cabi.call("tt_rmsnorm_backward_partials", s["dx"].data_ptr(), s["dy"].data_ptr(), s["x"].data_ptr(),
+                           self.p0.data_ptr(), self.ws.data_ptr(), self.ws.numel(), ctypes.byref(self.n_partials),
+                           self.rows, self.cols, self.w.eps, self.stream)
+
+    def reduce(self):
+        self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
+                       self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
+
+    def run(self, steps, warmup):
+        """Returns wall seconds per step and per-kernel mean microseconds from HIP events."""
+        torch = self.torch
+        # Untimed set-up: ~50 ms of the same launches so that the GPU has left its idle
+        # power state before the W warm-up steps (core clocks take tens of milliseconds to
+        # ramp, and the backward kernel is sensitive to them while they do).
+        t_ramp = time.perf_counter() + 0.05
+        while time.perf_counter() < t_ramp:
+            self.fwd(0); self.bwd_partials(0); self.reduce()
+            torch.cuda.synchronize()
+        for i in range(warmup):
+            self.fwd(i); self.bwd_partials(i); self.reduce()
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            e = ev[i]
+            e[0].record(); self.fwd(i)
+            e[1].record(); self.bwd_partials(i)
+            e[2].record(); self.reduce()
+            e[3].record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / steps
+        us = lambda a, b: [e[a].elapsed_time(e[b]) * 1e3 for e in ev]
+        return wall, {"fwd": us(0, 1), "bwd": us(1, 2), "reduce": us(2, 3)}
+
+
+def cpu_baseline(w, seconds):
+    """PyTorch-eager fwd + autograd bwd of the same op on the host CPU, bounded row sample."""
+    import torch
+    from oracle import eager_reference as E
+    from teletron_amd.workloads import make_inputs
+    threads = torch.get_num_threads()
+    sample_rows = min(w.shape[1], 16384)
+    t = make_inputs(w, seed=0, rows=sample_rows)
+    elements = t["x"].numel()
+    if w.op == "adaln":
+        fn = lambda: E.eager_adaln_fwd_bwd(t["x"], t["scale"], t["shift"], t["dy"], w.eps)
+    else:
+        fn = lambda: E.eager_rmsnorm_fwd_bwd(t["x"], t["gamma"], t["dy"], w.eps)
+    fn()
+    times = []
+    t_end = time.perf_counter() + seconds
+    while len(times) < 5 or time.perf_counter() < t_end:
+        t0 = time.perf_counter(); fn(); times.append(time.perf_counter() - t0)
+        if len(times) >= 2000:
+            break
+    med = statistics.median(times)
+    return {"value": round(10.0 * elements / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{w.op} eager bf16 fwd+autograd bwd on x{list(t['x'].shape)} (first {sample_rows} rows of the "
+                      f"workload), median of {len(times)} runs, {med * 1e3:.1f} ms/run, "
+                      f"{t['x'].numel() // w.cols / med:.3e} rows/s, 10 B/element"}
+
+
+def measure(w, steps, warmup):
+    g = GpuWorkload(w)
+    wall, k = g.run(steps, warmup)
+    bytes_step = w.algorithmic_bytes("fwd+bwd")
+    mean = lambda v: sum(v) / len(v)
+    res = {
+        "gbps": bytes_step / wall / 1e9,
+        "ms_per_step": wall * 1e3,
+        "rows_per_s": w.rows / wall,
+        "fwd_us": mean(k["fwd"]), "bwd_us": mean(k["bwd"]), "reduce_us": mean(k["reduce"]),
+        "fwd_gbps": w.algorithmic_bytes("fwd") / mean(k["fwd"]) / 1e3,
+        "bwd_gbps": w.algorithmic_bytes("bwd") / mean(k["bwd"]) / 1e3,
+        "n_partials": g.n_partials.value,
+    }
+    del g
+    import torch
+    torch.cuda.empty_cache()
+    return res
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}); rows are independent, so more GPUs "
+              "would each run this same kernel on a row shard. Re-run with --gpus 1.", file=sys.stderr)
+        return 2
+    import torch
+    from teletron_amd.workloads import WORKLOADS
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HIP kernels have no CPU fallback.", file=sys.stderr)
+        return 2
+    w = WORKLOADS[args.workload]
+    r = measure(w, args.steps, args.warmup)
+    out = {
+        "metric": METRIC, "value": round(r["gbps"], 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16_io_f32_math", "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.op} fwd+bwd, x{list(w.shape)} bf16, params{list(w.param_shape)} bf16, "
+                               f"eps {w.eps}; math in fp32, storage bf16",
+                   "buffer_sets": 2, "bytes_per_step": w.algorithmic_bytes("fwd+bwd")},
+        "pct_of_peak": round(100.0 * r["gbps"] / HBM_PEAK_GBPS, 2),
+        "rows_per_s": round(r["rows_per_s"], 1),
+        "kernels_us": {"forward": round(r["fwd_us"], 2), "backward_streaming": round(r["bwd_us"], 2),
+                       "reduce_partials": round(r["reduce_us"], 2)},
+        "roofline": {"bound": "hbm", "achieved": round(r["bwd_gbps"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(r["bwd_gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "norm_bwd_wide (backward streaming kernel)",
+                     "algorithmic_bytes_per_launch": w.algorithmic_bytes("bwd"),
+                     "forward_kernel": {"achieved": round(r["fwd_gbps"], 1),
+                                        "frac": round(r["fwd_gbps"] / HBM_PEAK_GBPS, 4),
+                                        "algorithmic_bytes_per_launch": w.algorithmic_bytes("fwd")}},
+    }
+    also = {}
+    for name in [n for n in args.also.split(",") if n and n != args.workload]:
+        wa = WORKLOADS[name]
+        ra = measure(wa, max(5, args.steps // 2), 3)
+        also[name] = {"value": round(ra["gbps"], 1), "unit": "GB/s", "pct_of_peak": round(100 * ra["gbps"] / HBM_PEAK_GBPS, 2),
+                      "ms_per_step": round(ra["ms_per_step"], 4), "forward_us": round(ra["fwd_us"], 2),
+                      "backward_streaming_us": round(ra["bwd_us"], 2), "reduce_partials_us": round(ra["reduce_us"], 2)}
+    if also:
+        out["also"] = also
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

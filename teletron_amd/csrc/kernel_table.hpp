@@ -11,6 +11,7 @@ struct KernelInfo {
   const void* fn;   // __global__ function taking one FwdArgs / BwdArgs by value
   int threads;      // workgroup size
   int tile_rows;    // rows one workgroup consumes per loop iteration
+  int lane_loads;   // 128-bit loads per lane and streamed tensor in one tile
 };
 
 // Wide variants: (index, W waves per row, P packs per lane).  A row of `packs`
@@ -31,7 +32,7 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 
 // ---- tuning constants (rows in flight per row group, row groups per workgroup)
 #ifndef TT_FWD_R
-#define TT_FWD_R 2
+#define TT_FWD_R 1
 #endif
 #ifndef TT_FWD_Q
 #define TT_FWD_Q 1
@@ -77,22 +78,22 @@ inline int select_narrow(int packs) {
 template <int KIND, int W, int P, bool FULL>
 KernelInfo info_fwd_wide() {
   constexpr int R = fwd_wide_R(W, P), Q = fwd_wide_Q(W, P);
-  return {reinterpret_cast<const void*>(&norm_fwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R};
+  return {reinterpret_cast<const void*>(&norm_fwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
 }
 template <int KIND, int W, int P, bool FULL>
 KernelInfo info_bwd_wide() {
   constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
-  return {reinterpret_cast<const void*>(&norm_bwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R};
+  return {reinterpret_cast<const void*>(&norm_bwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_fwd_narrow() {
   constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
-  return {reinterpret_cast<const void*>(&norm_fwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L)};
+  return {reinterpret_cast<const void*>(&norm_fwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_narrow() {
   constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
-  return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L)};
+  return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 
 template <int KIND>
@@ -110,7 +111,7 @@ KernelInfo lookup_fwd(bool narrow, int idx, bool full) {
 #undef X
     }
   }
-  return {nullptr, 0, 0};
+  return {nullptr, 0, 0, 0};
 }
 template <int KIND>
 KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
@@ -127,7 +128,7 @@ KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
 #undef X
     }
   }
-  return {nullptr, 0, 0};
+  return {nullptr, 0, 0, 0};
 }
 
 // Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, rms_fwd.hip, rms_bwd.hip).

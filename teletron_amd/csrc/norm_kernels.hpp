@@ -24,6 +24,12 @@ namespace tt {
 
 enum Kind : int { kAdaLN = 0, kRMS = 1 };
 
+// Software prefetch of the next tile (see the kernels); a build-time switch for A/B timing.
+#ifndef TT_PREFETCH
+#define TT_PREFETCH 1
+#endif
+constexpr bool PF = TT_PREFETCH != 0;
+
 struct FwdArgs {
   void* y;
   const void* x;
@@ -60,6 +66,9 @@ struct BwdArgs {
 // the reduction in between, which every wave reaches after its reads.
 template <int W, int NV>
 __device__ __forceinline__ void rowgroup_allsum(float (&v)[NV], float* buf, int w, int lane) {
+#ifdef TT_EXPERIMENT_NORED
+  return;
+#endif
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = wave_allsum(v[i]);
   if constexpr (W > 1) {
@@ -113,21 +122,36 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
     }
   }
 
+  // Raw packs of the tile being fetched.  With PF the loads of the next tile are
+  // issued before the arithmetic of the current one, so every wave keeps a tile
+  // in flight while it computes.
+  u32x4 raw[R][P];
+  auto fetch = [&](int64_t t) {
+    const int64_t r0 = t * (Q * R) + q * R;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        raw[r][p] = u32x4{0, 0, 0, 0};
+        if (r0 + r < S && act[p]) raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
+      }
+  };
+
   unsigned phase = 0;
-  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t row0 = tile * (Q * R) + q * R;
     float xf[R][P][8];
     bool rv[R];
+    if (!PF) fetch(tile);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       rv[r] = row0 + r < S;
 #pragma unroll
-      for (int p = 0; p < P; ++p) {
-        u32x4 raw = {0, 0, 0, 0};
-        if (rv[r] && act[p]) raw = load_stream(a.x, (size_t)((b * S + row0 + r) * C + col[p]));
-        unpack8(raw, xf[r][p]);
-      }
+      for (int p = 0; p < P; ++p) unpack8(raw[r][p], xf[r][p]);
     }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 
     float mean[R];
 #pragma unroll
@@ -234,26 +258,41 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
     }
   }
 
+  u32x4 rawx[R][P], rawd[R][P];
+  auto fetch = [&](int64_t t) {
+    const int64_t r0 = t * (Q * R) + q * R;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        rawx[r][p] = u32x4{0, 0, 0, 0};
+        rawd[r][p] = u32x4{0, 0, 0, 0};
+        if (r0 + r < S && act[p]) {
+          const size_t off = (size_t)((b * S + r0 + r) * C + col[p]);
+          rawx[r][p] = load_stream(a.x, off);
+          rawd[r][p] = load_stream(a.dy, off);
+        }
+      }
+  };
+
   unsigned phase = 0;
-  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t row0 = tile * (Q * R) + q * R;
     float xf[R][P][8], df[R][P][8];
     bool rv[R];
+    if (!PF) fetch(tile);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       rv[r] = row0 + r < S;
 #pragma unroll
       for (int p = 0; p < P; ++p) {
-        u32x4 rx = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
-        if (rv[r] && act[p]) {
-          const size_t off = (size_t)((b * S + row0 + r) * C + col[p]);
-          rx = load_stream(a.x, off);
-          rd = load_stream(a.dy, off);
-        }
-        unpack8(rx, xf[r][p]);
-        unpack8(rd, df[r][p]);
+        unpack8(rawx[r][p], xf[r][p]);
+        unpack8(rawd[r][p], df[r][p]);
       }
     }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 
     float mean[R];
 #pragma unroll
@@ -402,18 +441,30 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
     }
   }
 
-  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+  u32x4 raw[R];
+  auto fetch = [&](int64_t t) {
+    const int64_t rb = t * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t rr = rb + r * RPW;
+      raw[r] = u32x4{0, 0, 0, 0};
+      if (rr < S && act) raw[r] = load_stream(a.x, (size_t)((b * S + rr) * C + col));
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
     float xf[R][8];
     bool rv[R];
+    if (!PF) fetch(tile);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int64_t rr = rbase + r * RPW;
-      rv[r] = rr < S;
-      u32x4 raw = {0, 0, 0, 0};
-      if (rv[r] && act) raw = load_stream(a.x, (size_t)((b * S + rr) * C + col));
-      unpack8(raw, xf[r]);
+      rv[r] = rbase + r * RPW < S;
+      unpack8(raw[r], xf[r]);
     }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float mean = 0.f;
@@ -485,23 +536,36 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
     }
   }
 
-  for (int64_t tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+  u32x4 rawx[R], rawd[R];
+  auto fetch = [&](int64_t t) {
+    const int64_t rb = t * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t rr = rb + r * RPW;
+      rawx[r] = u32x4{0, 0, 0, 0};
+      rawd[r] = u32x4{0, 0, 0, 0};
+      if (rr < S && act) {
+        const size_t off = (size_t)((b * S + rr) * C + col);
+        rawx[r] = load_stream(a.x, off);
+        rawd[r] = load_stream(a.dy, off);
+      }
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
     float xf[R][8], df[R][8];
     bool rv[R];
+    if (!PF) fetch(tile);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int64_t rr = rbase + r * RPW;
-      rv[r] = rr < S;
-      u32x4 rx = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
-      if (rv[r] && act) {
-        const size_t off = (size_t)((b * S + rr) * C + col);
-        rx = load_stream(a.x, off);
-        rd = load_stream(a.dy, off);
-      }
-      unpack8(rx, xf[r]);
-      unpack8(rd, df[r]);
+      rv[r] = rbase + r * RPW < S;
+      unpack8(rawx[r], xf[r]);
+      unpack8(rawd[r], df[r]);
     }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float mean = 0.f;
