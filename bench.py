@@ -29,6 +29,12 @@ REPO_ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, REPO_ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E peak
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled against a plain copy of
+# known size); the counters cannot be read from inside this process, so the measured figures are
+# carried here.  Valid only while the backward kernel writes the stated number of partial sums.
+MEASURED_TRAFFIC_BYTES = {
+    "adaln_wan14b": {"fwd": 1548465816, "bwd": 2343470191, "n_partials": 512},
+}
 METRIC = "fwd+bwd HBM GB/s and % of peak, AdaLN/RMSNorm at Wan-14B shape 75600x5120"
 
 
@@ -41,6 +47,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
     ap.add_argument("--also", default="rmsnorm_wan14b_qk", help="comma list of further workloads reported under 'also'")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
+                         "that hardware byte counters collected over this run can be scaled against it")
     return ap.parse_args()
 
 
@@ -195,6 +204,8 @@ def main():
         return 2
     w = WORKLOADS[args.workload]
     r = measure(w, args.steps, args.warmup)
+    mt = MEASURED_TRAFFIC_BYTES.get(w.name)
+    traffic = mt["bwd"] if mt and mt["n_partials"] == r["n_partials"] else None
     out = {
         "metric": METRIC, "value": round(r["gbps"], 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 4),
@@ -207,7 +218,7 @@ def main():
         "kernels_us": {"forward": round(r["fwd_us"], 2), "backward_streaming": round(r["bwd_us"], 2),
                        "reduce_partials": round(r["reduce_us"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(r["bwd_gbps"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(r["bwd_gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(r["bwd_gbps"] / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "kernel": "norm_bwd_wide (backward streaming kernel)",
                      "algorithmic_bytes_per_launch": w.algorithmic_bytes("bwd"),
                      "forward_kernel": {"achieved": round(r["fwd_gbps"], 1),
@@ -223,6 +234,13 @@ def main():
                       "backward_streaming_us": round(ra["bwd_us"], 2), "reduce_partials_us": round(ra["reduce_us"], 2)}
     if also:
         out["also"] = also
+    if args.calibrate_copy:
+        src = torch.empty(w.elements, dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration_copy_bytes"] = src.numel() * 2
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
     print(json.dumps(out))

@@ -66,9 +66,6 @@ struct BwdArgs {
 // the reduction in between, which every wave reaches after its reads.
 template <int W, int NV>
 __device__ __forceinline__ void rowgroup_allsum(float (&v)[NV], float* buf, int w, int lane) {
-#ifdef TT_EXPERIMENT_NORED
-  return;
-#endif
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = wave_allsum(v[i]);
   if constexpr (W > 1) {
