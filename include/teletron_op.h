@@ -129,6 +129,43 @@ TT_API int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x,
 TT_API int tt_reduce_partials(float* out0, float* out1, const void* workspace,
                        int n_batches, int n_partials, int n_acc, int64_t cols, void* stream);
 
+/* ------------------------------------------------------------------ reference-compatible contract
+ * Argument for argument the launchers the reference's pybind glue calls, plus a trailing
+ * stream (the reference launches on the legacy default stream) and, for backward, the
+ * workspace the reference allocates on the fly (weight_backward.cu:229).  They keep the
+ * reference's saved tensors and output types:
+ *   - forward also writes x_norm = bf16((x - mean) * rstd) and inv_variance = rstd [rows] fp32;
+ *   - AdaLN backward reads x_norm and inv_variance (not x); scale/shift are one [cols]
+ *     vector; dscale/dshift are bf16 [cols];
+ *   - RMSNorm backward reads the forward *output* and reconstructs x_hat = y / weight, so a
+ *     zero weight gives Inf/NaN exactly as in the reference; dweight is bf16 [cols].
+ * Unlike the reference, any cols that is a multiple of 8 (up to TT_MAX_COLS) is accepted,
+ * the arithmetic is fp32 with one rounding at each store, and parameter gradients are
+ * reduced in fp32 before the single rounding to bf16.
+ */
+
+/* launch_adaln_forward: adaln_kernel.h:21-30, adaln_forward.cu:198-220, called from adaln_ops.cpp:16-26. */
+TT_API int tt_launch_adaln_forward(void* output, void* x_norm, const void* input,
+                                   const void* scale, const void* shift,
+                                   int64_t rows, int64_t cols, double epsilon,
+                                   float* inv_variance, void* stream);
+/* launch_adaln_backward: adaln_kernel.h:37-46, adaln_backward.cu:129-151, called from adaln_ops.cpp:39-49.
+ * Workspace: tt_adaln_backward_workspace_bytes(rows, cols, rows). */
+TT_API int tt_launch_adaln_backward(void* dinp, void* dscale, void* dshift,
+                                    const void* dout, const void* x_norm, const void* scale,
+                                    const float* inv_variance, int64_t rows, int64_t cols,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+/* launch_rms_forward: rmsnorm_kernel.h:5-12, rms_forward.cu:102-121, called from rms_ops.cpp:14-22. */
+TT_API int tt_launch_rms_forward(void* output, const void* input, const void* weight,
+                                 int64_t rows, int64_t cols, double epsilon,
+                                 float* inv_variance, void* stream);
+/* launch_rms_backward: rmsnorm_kernel.h:19-25, rms_backward.cu:91-112, called from rms_ops.cpp:34-43.
+ * x_rmsnorm is the forward output.  Workspace: tt_rmsnorm_backward_workspace_bytes(rows, cols). */
+TT_API int tt_launch_rms_backward(void* dinp, void* dweight,
+                                  const void* dout, const void* x_rmsnorm, const void* weight,
+                                  const float* inv_variance, int64_t rows, int64_t cols,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

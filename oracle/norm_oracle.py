@@ -142,6 +142,38 @@ def rmsnorm_backward(dy, x, gamma, eps: float):
     return dx, dgamma
 
 
+# --------------------------------------------------------------------------- reference contract (saved tensors)
+def adaln_backward_from_saved(dy, x_norm, scale, rstd):
+    """AdaLN backward as the reference's kernels receive it: the saved ``x_norm`` (= x_hat as
+    stored by forward) and per-row ``rstd`` instead of x (adaln_backward.cu:85-125,
+    scale_shift_backward.cu:84-92).  One modulation vector ``scale[C]``.
+    Returns ``(dx, dscale[C], dshift[C])`` in float64."""
+    c = x_norm.shape[-1]
+    xh = _f64(x_norm).reshape(-1, c)
+    dyf = _f64(dy).reshape(-1, c)
+    r = _f64(rstd).reshape(-1, 1)
+    g = dyf * (1.0 + _f64(scale).reshape(1, c))
+    m1 = g.mean(dim=-1, keepdim=True)
+    m2 = (g * xh).mean(dim=-1, keepdim=True)
+    dx = r * (g - m1 - xh * m2)
+    return dx.reshape(x_norm.shape), (dyf * xh).sum(dim=0), dyf.sum(dim=0)
+
+
+def rmsnorm_backward_from_saved(dy, y, gamma, rstd):
+    """RMSNorm backward as the reference's kernels receive it: the saved forward output ``y``
+    and per-row ``rstd``; x_hat is reconstructed as y / gamma (rms_backward.cu:64-87,
+    weight_backward.cu:84-103).  Returns ``(dx, dgamma[C])`` in float64."""
+    c = y.shape[-1]
+    w = _f64(gamma).reshape(1, c)
+    xh = _f64(y).reshape(-1, c) / w
+    dyf = _f64(dy).reshape(-1, c)
+    r = _f64(rstd).reshape(-1, 1)
+    g = dyf * w
+    m2 = (g * xh).mean(dim=-1, keepdim=True)
+    dx = r * (g - xh * m2)
+    return dx.reshape(y.shape), (dyf * xh).sum(dim=0)
+
+
 # --------------------------------------------------------------------------- chunked variants
 def adaln_backward_param_grads_chunked(dy, x, eps: float, n_batches: int = 1, chunk_rows: int = 4096):
     """dscale / dshift only, streamed over row chunks so that full-size shapes

@@ -4,9 +4,18 @@ The compute path is hand-written HIP for gfx950 in ``libteletron_op.so`` (C ABI,
 ``include/teletron_op.h``); Python only validates, allocates and launches.
 """
 from .functional import (AdaLNModelFunction, FusedAdaLN, FusedRMSNorm, RMSNormModelFunction,
-                         fused_adaln, fused_rmsnorm)
+                         adaln_modulate, rms_norm)
 from . import cabi, ops, workloads
 
 __all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "FusedAdaLN", "FusedRMSNorm",
-           "fused_adaln", "fused_rmsnorm", "cabi", "ops", "workloads"]
+           "adaln_modulate", "rms_norm", "cabi", "ops", "workloads", "install_reference_modules"]
+
+
+def install_reference_modules() -> None:
+    """Make ``import fused_adaln`` / ``import fused_rmsnorm`` (the reference's top-level module
+    names, ``teletron_op/README.md:55,133``) resolve to this package's glue modules."""
+    import importlib
+    import sys
+    for name in ("fused_adaln", "fused_rmsnorm"):
+        sys.modules.setdefault(name, importlib.import_module(f"{__name__}.{name}"))
 __version__ = "0.1.0"

@@ -19,7 +19,8 @@ CSRC = PKG_DIR / "csrc"
 OBJ_DIR = CSRC / "build"
 LIB_PATH = PKG_DIR / "libteletron_op.so"
 
-HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_bwd.hip", "rms_fwd.hip", "rms_bwd.hip"]
+HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_bwd.hip", "adaln_bwd_saved.hip",
+               "rms_fwd.hip", "rms_bwd.hip", "rms_bwd_saved.hip"]
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form
 # v_pk_{add,mul,fma}_f32 from the scalar float code of these kernels.
@@ -71,13 +72,61 @@ def build_library(force: bool = True, defines=(), jobs: int = 8, verbose: bool =
     return LIB_PATH
 
 
+TORCH_EXT_MODULES = ["fused_adaln", "fused_rmsnorm"]
+
+
+def torch_ext_path(name: str) -> Path:
+    import sysconfig
+    return PKG_DIR / (name + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_torch_extensions(force: bool = True, verbose: bool = True):
+    """Compile the pybind / TORCH_LIBRARY glue modules (host C++ only, g++) against the
+    installed torch and link them to libteletron_op.so.  They hold no kernels."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+    if not LIB_PATH.exists():
+        build_library(force=True, verbose=verbose)
+    src_dir = CSRC / "torch_ext"
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    incs = []
+    for d in ce.include_paths("cuda") + [sysconfig.get_paths()["include"], str(REPO_ROOT / "include"), str(src_dir)]:
+        incs += ["-I", d]
+    abi = int(getattr(torch._C, "_GLIBCXX_USE_CXX11_ABI", True))
+    cxx = shutil.which("g++") or "g++"
+
+    def compile_one(name: str) -> Path:
+        src = src_dir / (name + ".cpp")
+        out = torch_ext_path(name)
+        deps = [src, src_dir / "glue.hpp", REPO_ROOT / "include" / "teletron_op.h"]
+        if not force and out.exists() and out.stat().st_mtime > max(d.stat().st_mtime for d in deps):
+            return out
+        cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+               f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+               f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-deprecated-declarations", *incs, str(src), "-o", str(out),
+               f"-L{torch_lib}", "-L/opt/rocm/lib", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip",
+               "-ltorch_hip", "-lamdhip64", str(LIB_PATH),
+               "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}", "-Wl,-rpath,/opt/rocm/lib"]
+        if verbose:
+            print("[teletron_amd.build] g++", src.name, flush=True)
+        _run(cmd)
+        return out
+
+    with ThreadPoolExecutor(max_workers=2) as pool:
+        return list(pool.map(compile_one, TORCH_EXT_MODULES))
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--force", action="store_true", help="recompile even if objects look current")
     ap.add_argument("--define", action="append", default=[], help="extra -D for hipcc (tuning constants)")
+    ap.add_argument("--no-torch-ext", action="store_true", help="skip the pybind/TORCH_LIBRARY glue modules")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     args = ap.parse_args(argv)
     build_library(force=args.force or bool(args.define), defines=args.define, jobs=args.jobs)
+    if not args.no_torch_ext:
+        build_torch_extensions(force=args.force)
     return 0
 
 

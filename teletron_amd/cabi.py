@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p, POINTER
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p, POINTER
 from pathlib import Path
 
 LIB_NAME = "libteletron_op.so"
@@ -52,6 +52,13 @@ PROTOTYPES = {
                                              c_void_p, c_size_t, POINTER(c_int),
                                              c_int64, c_int64, c_float, c_void_p]),
     "tt_reduce_partials": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
+    "tt_launch_adaln_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_int64, c_double, c_void_p, c_void_p]),
+    "tt_launch_adaln_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "tt_launch_rms_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_double, c_void_p, c_void_p]),
+    "tt_launch_rms_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
 }
 
 _lib = None

@@ -72,7 +72,7 @@ struct Plan {
   int packs = 0;
 };
 
-enum Dir { kFwd, kBwd };
+enum Dir { kFwd, kBwd, kBwdSaved };
 
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
 constexpr int kMaxWgsPerCu = 8;
@@ -90,8 +90,12 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   const int slots = narrow ? kNarrowL[idx] : 64 * kWideW[idx] * kWideP[idx];
   const bool full = (slots == packs);
   KernelInfo k;
-  if (kind == kAdaLN) k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full) : adaln_bwd_kernel(narrow, idx, full);
-  else                k = dir == kFwd ? rms_fwd_kernel(narrow, idx, full) : rms_bwd_kernel(narrow, idx, full);
+  if (kind == kAdaLN)
+    k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
+      : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
+  else
+    k = dir == kFwd ? rms_fwd_kernel(narrow, idx, full)
+      : dir == kBwd ? rms_bwd_kernel(narrow, idx, full) : rms_bwd_saved_kernel(narrow, idx, full);
   if (!k.fn) return TT_ERR_UNSUPPORTED;
 
   int cus = 0, per_cu = 0;
@@ -151,16 +155,16 @@ int launch(const Plan& p, Args& args, void* stream) {
   return TT_OK;
 }
 
-int forward(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd,
+int forward(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd, void* x_norm,
             int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
   if (rows == 0) return TT_OK;
   if (!y || !x || !p0 || (kind == kAdaLN && !p1)) return TT_ERR_INVALID_ARGUMENT;
-  if (!aligned16(y) || !aligned16(x) || !aligned16(p0) || !aligned16(p1)) return TT_ERR_UNSUPPORTED;
+  if (!aligned16(y) || !aligned16(x) || !aligned16(p0) || !aligned16(p1) || !aligned16(x_norm)) return TT_ERR_UNSUPPORTED;
   Plan p;
   int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p);
   if (rc != TT_OK) return rc;
   FwdArgs a;
-  a.y = y; a.x = x; a.p0 = p0; a.p1 = p1; a.mean = mean; a.rstd = rstd;
+  a.y = y; a.x = x; a.p0 = p0; a.p1 = p1; a.mean = mean; a.rstd = rstd; a.x_norm = x_norm;
   a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
   a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
   return launch(p, a, stream);
@@ -187,8 +191,29 @@ int backward_partials(int kind, void* dx, const void* dy, const void* x, const v
   return rc;
 }
 
-int reduce(float* out0, float* out1, const void* workspace, int n_batches, int n_partials, int n_acc,
-           int64_t cols, void* stream) {
+int backward_saved_partials(int kind, void* dx, const void* dy, const void* xs, const void* p0, const float* rstd,
+                            void* workspace, size_t workspace_bytes, int* n_partials,
+                            int64_t rows, int64_t cols, void* stream) {
+  *n_partials = 0;
+  if (rows == 0) return TT_OK;
+  if (!dx || !dy || !xs || !p0 || !rstd) return TT_ERR_INVALID_ARGUMENT;
+  if (!aligned16(dx) || !aligned16(dy) || !aligned16(xs) || !aligned16(p0)) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kind, kBwdSaved, rows, cols, rows, &p);
+  if (rc != TT_OK) return rc;
+  const int n_acc = kind == kAdaLN ? 2 : 1;
+  if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;
+  BwdSavedArgs a;
+  a.dx = dx; a.dy = dy; a.xs = xs; a.p0 = p0; a.rstd = rstd; a.partials = static_cast<float*>(workspace);
+  a.rows_per_batch = rows; a.n_tiles = p.n_tiles;
+  a.cols = (int)cols; a.packs = p.packs; a.inv_cols = 1.0f / (float)cols;
+  rc = launch(p, a, stream);
+  if (rc == TT_OK) *n_partials = p.grid_x;
+  return rc;
+}
+
+int reduce(void* out0, void* out1, const void* workspace, int n_batches, int n_partials, int n_acc,
+           int64_t cols, bool out_bf16, void* stream) {
   if (n_batches == 0) return TT_OK;
   if (!out0 || !workspace || n_batches < 0 || n_batches > 65535 || n_partials <= 0 || cols <= 0 ||
       cols > TT_MAX_COLS || (n_acc != 1 && n_acc != 2) || (n_acc == 2 && !out1))
@@ -196,8 +221,9 @@ int reduce(float* out0, float* out1, const void* workspace, int n_batches, int n
   const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)n_batches, 1);
   const float* ws = static_cast<const float*>(workspace);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (n_acc == 2) hipLaunchKernelGGL(reduce_partials<2>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols);
-  else            hipLaunchKernelGGL(reduce_partials<1>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols);
+  const int bf = out_bf16 ? 1 : 0;
+  if (n_acc == 2) hipLaunchKernelGGL(reduce_partials<2>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols, bf);
+  else            hipLaunchKernelGGL(reduce_partials<1>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols, bf);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return TT_OK;
@@ -231,12 +257,12 @@ TT_API void tt_debug_set_wgs_per_cu(int n) { g_wgs_per_cu_override.store(n < 0 ?
 
 int tt_adaln_forward(void* y, const void* x, const void* scale, const void* shift, float* mean, float* rstd,
                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
-  return forward(kAdaLN, y, x, scale, shift, mean, rstd, rows, cols, rows_per_batch, eps, stream);
+  return forward(kAdaLN, y, x, scale, shift, mean, rstd, nullptr, rows, cols, rows_per_batch, eps, stream);
 }
 
 int tt_rmsnorm_forward(void* y, const void* x, const void* weight, float* rstd,
                        int64_t rows, int64_t cols, float eps, void* stream) {
-  return forward(kRMS, y, x, weight, nullptr, nullptr, rstd, rows, cols, rows, eps, stream);
+  return forward(kRMS, y, x, weight, nullptr, nullptr, rstd, nullptr, rows, cols, rows, eps, stream);
 }
 
 size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch) {
@@ -261,7 +287,7 @@ int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x, const 
 
 int tt_reduce_partials(float* out0, float* out1, const void* workspace,
                        int n_batches, int n_partials, int n_acc, int64_t cols, void* stream) {
-  return reduce(out0, out1, workspace, n_batches, n_partials, n_acc, cols, stream);
+  return reduce(out0, out1, workspace, n_batches, n_partials, n_acc, cols, false, stream);
 }
 
 int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, const void* x, const void* scale,
@@ -273,7 +299,7 @@ int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, co
   int rc = backward_partials(kAdaLN, dx, dy, x, scale, workspace, workspace_bytes, &n_partials,
                              rows, cols, rows_per_batch, eps, stream);
   if (rc != TT_OK) return rc;
-  return reduce(dscale, dshift, workspace, (int)(rows / rows_per_batch), n_partials, 2, cols, stream);
+  return reduce(dscale, dshift, workspace, (int)(rows / rows_per_batch), n_partials, 2, cols, false, stream);
 }
 
 int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
@@ -285,7 +311,46 @@ int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x,
   int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
                              rows, cols, rows, eps, stream);
   if (rc != TT_OK) return rc;
-  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, stream);
+  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, false, stream);
+}
+
+// ---------------------------------------------------------------- reference-compatible contract
+int tt_launch_adaln_forward(void* output, void* x_norm, const void* input, const void* scale, const void* shift,
+                            int64_t rows, int64_t cols, double epsilon, float* inv_variance, void* stream) {
+  if (rows != 0 && (!x_norm || !inv_variance)) return TT_ERR_INVALID_ARGUMENT;
+  return forward(kAdaLN, output, input, scale, shift, nullptr, inv_variance, x_norm, rows, cols, rows,
+                 static_cast<float>(epsilon), stream);
+}
+
+int tt_launch_adaln_backward(void* dinp, void* dscale, void* dshift, const void* dout, const void* x_norm,
+                             const void* scale, const float* inv_variance, int64_t rows, int64_t cols,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dscale || !dshift) return TT_ERR_INVALID_ARGUMENT;
+  int n_partials = 0;
+  int rc = backward_saved_partials(kAdaLN, dinp, dout, x_norm, scale, inv_variance, workspace, workspace_bytes,
+                                   &n_partials, rows, cols, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dscale, dshift, workspace, 1, n_partials, 2, cols, true, stream);
+}
+
+int tt_launch_rms_forward(void* output, const void* input, const void* weight, int64_t rows, int64_t cols,
+                          double epsilon, float* inv_variance, void* stream) {
+  if (rows != 0 && !inv_variance) return TT_ERR_INVALID_ARGUMENT;
+  return forward(kRMS, output, input, weight, nullptr, nullptr, inv_variance, nullptr, rows, cols, rows,
+                 static_cast<float>(epsilon), stream);
+}
+
+int tt_launch_rms_backward(void* dinp, void* dweight, const void* dout, const void* x_rmsnorm, const void* weight,
+                           const float* inv_variance, int64_t rows, int64_t cols,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dweight) return TT_ERR_INVALID_ARGUMENT;
+  int n_partials = 0;
+  int rc = backward_saved_partials(kRMS, dinp, dout, x_rmsnorm, weight, inv_variance, workspace, workspace_bytes,
+                                   &n_partials, rows, cols, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, true, stream);
 }
 
 }  // extern "C"

@@ -85,6 +85,16 @@ KernelInfo info_bwd_wide() {
   constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
   return {reinterpret_cast<const void*>(&norm_bwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
 }
+template <int KIND, int W, int P, bool FULL>
+KernelInfo info_bwd_saved_wide() {
+  constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_bwd_saved_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
+}
+template <int KIND, int L, bool FULL>
+KernelInfo info_bwd_saved_narrow() {
+  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&norm_bwd_saved_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
+}
 template <int KIND, int L, bool FULL>
 KernelInfo info_fwd_narrow() {
   constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
@@ -131,10 +141,30 @@ KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
-// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, rms_fwd.hip, rms_bwd.hip).
+template <int KIND>
+KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L) case i: return full ? info_bwd_saved_narrow<KIND, L, true>() : info_bwd_saved_narrow<KIND, L, false>();
+      TT_NARROW_LIST(X)
+#undef X
+    }
+  } else {
+    switch (idx) {
+#define X(i, W, P) case i: return full ? info_bwd_saved_wide<KIND, W, P, true>() : info_bwd_saved_wide<KIND, W, P, false>();
+      TT_WIDE_LIST(X)
+#undef X
+    }
+  }
+  return {nullptr, 0, 0, 0};
+}
+
+// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip).
 KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
+KernelInfo adaln_bwd_saved_kernel(bool narrow, int idx, bool full);
+KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
 
 }  // namespace tt

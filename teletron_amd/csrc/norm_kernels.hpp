@@ -37,6 +37,7 @@ struct FwdArgs {
   const void* p1;   // AdaLN: shift [B, C];  RMSNorm: unused
   float* mean;      // optional [rows]
   float* rstd;      // optional [rows]
+  void* x_norm;     // optional [rows, cols] bf16: the normalised input before modulation (AdaLN)
   int64_t rows_per_batch;
   int64_t n_tiles;  // tiles per batch
   int cols;
@@ -199,18 +200,71 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
 #pragma unroll
         for (int p = 0; p < P; ++p) {
           if (act[p]) {
-            float o[8];
+            float o[8], n[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const float xh = xf[r][p][j] * rstd;
+              n[j] = xh;
               o[j] = ADALN ? fmaf(xh, g[p][j], sh[p][j]) : xh * g[p][j];
             }
             store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
+            if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col[p]), pack8(n));
           }
         }
         if (w == 0 && lane == 0) {
           if (ADALN && a.mean) a.mean[row] = mean[r];
           if (a.rstd) a.rstd[row] = rstd;
+        }
+      }
+    }
+  }
+}
+
+// Epilogue of the wide backward kernels: fold the Q row groups of the workgroup into
+// group 0 (in group order, through LDS) and write the workgroup's partial column sums.
+template <bool ADALN, int W, int P, int Q>
+__device__ __forceinline__ void wide_write_partials(float (&acc0)[P][8], float (&acc1)[P][8], const bool (&act)[P],
+                                                    const int (&col)[P], float* partials, int64_t b, int C,
+                                                    int q, int w, int lane) {
+  constexpr int NACC = ADALN ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) float comb[Q > 1 ? 64 * W * P * 8 : 4];
+  if constexpr (Q > 1) {
+#pragma unroll
+    for (int acc = 0; acc < NACC; ++acc) {
+      for (int qq = 1; qq < Q; ++qq) {
+        __syncthreads();
+        if (q == qq) {
+#pragma unroll
+          for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              comb[((p * W + w) * 64 + lane) * 8 + j] = acc == 0 ? acc0[p][j] : acc1[p][j];
+        }
+        __syncthreads();
+        if (q == 0) {
+#pragma unroll
+          for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float t = comb[((p * W + w) * 64 + lane) * 8 + j];
+              if (acc == 0) acc0[p][j] += t; else acc1[p][j] += t;
+            }
+        }
+      }
+    }
+  }
+  if (q == 0) {
+    float* base = partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      if (act[p]) {
+        f32x4* d0 = reinterpret_cast<f32x4*>(base + col[p]);
+        d0[0] = f32x4{acc0[p][0], acc0[p][1], acc0[p][2], acc0[p][3]};
+        d0[1] = f32x4{acc0[p][4], acc0[p][5], acc0[p][6], acc0[p][7]};
+        if constexpr (ADALN) {
+          f32x4* d1 = reinterpret_cast<f32x4*>(base + C + col[p]);
+          d1[0] = f32x4{acc1[p][0], acc1[p][1], acc1[p][2], acc1[p][3]};
+          d1[1] = f32x4{acc1[p][4], acc1[p][5], acc1[p][6], acc1[p][7]};
         }
       }
     }
@@ -224,7 +278,6 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
   constexpr int NACC = ADALN ? 2 : 1;
   constexpr int NV = ADALN ? 3 : 2;  // reduced values per row in the main phase
   __shared__ float red[2][Q][W * R * NV];
-  __shared__ __attribute__((aligned(16))) float comb[Q > 1 ? 64 * W * P * 8 : 4];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -361,49 +414,7 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
     }
   }
 
-  // Fold the Q row groups of this workgroup into group 0, in group order.
-  if constexpr (Q > 1) {
-#pragma unroll
-    for (int acc = 0; acc < NACC; ++acc) {
-      for (int qq = 1; qq < Q; ++qq) {
-        __syncthreads();
-        if (q == qq) {
-#pragma unroll
-          for (int p = 0; p < P; ++p)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              comb[((p * W + w) * 64 + lane) * 8 + j] = acc == 0 ? acc0[p][j] : acc1[p][j];
-        }
-        __syncthreads();
-        if (q == 0) {
-#pragma unroll
-          for (int p = 0; p < P; ++p)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float t = comb[((p * W + w) * 64 + lane) * 8 + j];
-              if (acc == 0) acc0[p][j] += t; else acc1[p][j] += t;
-            }
-        }
-      }
-    }
-  }
-
-  if (q == 0) {
-    float* base = a.partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-      if (act[p]) {
-        f32x4* d0 = reinterpret_cast<f32x4*>(base + col[p]);
-        d0[0] = f32x4{acc0[p][0], acc0[p][1], acc0[p][2], acc0[p][3]};
-        d0[1] = f32x4{acc0[p][4], acc0[p][5], acc0[p][6], acc0[p][7]};
-        if constexpr (ADALN) {
-          f32x4* d1 = reinterpret_cast<f32x4*>(base + C + col[p]);
-          d1[0] = f32x4{acc1[p][0], acc1[p][1], acc1[p][2], acc1[p][3]};
-          d1[1] = f32x4{acc1[p][4], acc1[p][5], acc1[p][6], acc1[p][7]};
-        }
-      }
-    }
-  }
+  wide_write_partials<ADALN, W, P, Q>(acc0, acc1, act, col, a.partials, b, C, q, w, lane);
 }
 
 // ============================================================================ narrow forward
@@ -486,18 +497,56 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
       const float rstd = rsqrtf(v * a.inv_cols + a.eps);
       if (rv[r] && act) {
         const int64_t row = b * S + rbase + r * RPW;
-        float o[8];
+        float o[8], n[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float xh = xf[r][j] * rstd;
+          n[j] = xh;
           o[j] = ADALN ? fmaf(xh, g[j], sh[j]) : xh * g[j];
         }
         store_stream(a.y, (size_t)(row * C + col), pack8(o));
+        if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col), pack8(n));
         if (pi == 0) {
           if (ADALN && a.mean) a.mean[row] = mean;
           if (a.rstd) a.rstd[row] = rstd;
         }
       }
+    }
+  }
+}
+
+// Epilogue of the narrow backward kernels: fold the 64/L row slots of each wave (lanes
+// with equal pack index), then the waves through LDS, and write the partial column sums.
+template <bool ADALN, int L, int NW>
+__device__ __forceinline__ void narrow_write_partials(float (&acc0)[8], float (&acc1)[8], float* partials,
+                                                      int64_t b, int C, int pi, int ri, int wave) {
+  constexpr int NACC = ADALN ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) float comb[NW][NACC][L * 8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+#pragma unroll
+    for (int m = L; m < 64; m <<= 1) {
+      acc0[j] += __shfl_xor(acc0[j], m, 64);
+      if constexpr (ADALN) acc1[j] += __shfl_xor(acc1[j], m, 64);
+    }
+  }
+  if (ri == 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      comb[wave][0][pi * 8 + j] = acc0[j];
+      if constexpr (ADALN) comb[wave][NACC - 1][pi * 8 + j] = acc1[j];
+    }
+  }
+  __syncthreads();
+  float* base = partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
+  for (int i = threadIdx.x; i < NACC * L * 8; i += 64 * NW) {
+    const int acc = i / (L * 8);
+    const int c = i - acc * (L * 8);
+    if (c < C) {
+      float t = comb[0][acc][c];
+#pragma unroll
+      for (int ww = 1; ww < NW; ++ww) t += comb[ww][acc][c];
+      base[(size_t)acc * C + c] = t;
     }
   }
 }
@@ -508,7 +557,6 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
   constexpr int NACC = ADALN ? 2 : 1;
   constexpr int RPW = 64 / L;
-  __shared__ __attribute__((aligned(16))) float comb[NW][NACC][L * 8];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -605,43 +653,244 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
     }
   }
 
-  // Fold the 64/L row slots of the wave (lanes with equal pi), then the waves.
+  narrow_write_partials<ADALN, L, NW>(acc0, acc1, a.partials, b, C, pi, ri, wave);
+}
+
+
+// ============================================================================ backward from saved tensors
+// The reference's contract: backward receives the tensor saved by forward (AdaLN: x_norm,
+// RMSNorm: the forward output y, from which x_hat = y / weight) and the per-row rstd,
+// instead of x.  Same skeleton as above without the statistics phases.
+struct BwdSavedArgs {
+  void* dx;
+  const void* dy;
+  const void* xs;      // AdaLN: x_norm [rows, cols];  RMSNorm: forward output y [rows, cols]
+  const void* p0;      // AdaLN: scale [B, C];  RMSNorm: weight [C]
+  const float* rstd;   // [rows]
+  float* partials;
+  int64_t rows_per_batch;
+  int64_t n_tiles;
+  int cols;
+  int packs;
+  float inv_cols;
+};
+
+template <int KIND, int W, int P, int R, int Q, bool FULL>
+__global__ __launch_bounds__(64 * W * Q) void norm_bwd_saved_wide(const BwdSavedArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  constexpr int NV = ADALN ? 2 : 1;
+  __shared__ float red[2][Q][W * R * NV];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int q = wave / W;
+  const int w = wave - q * W;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+
+  int col[P];
+  bool act[P];
+  float g[P][8];    // 1 + scale, or weight
+  float gi[P][8];   // RMSNorm: 1 / weight (x_hat = y / weight); 0 on masked lanes
+  float acc0[P][8], acc1[P][8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-#pragma unroll
-    for (int m = L; m < 64; m <<= 1) {
-      acc0[j] += __shfl_xor(acc0[j], m, 64);
-      if constexpr (ADALN) acc1[j] += __shfl_xor(acc1[j], m, 64);
-    }
-  }
-  if (ri == 0) {
+  for (int p = 0; p < P; ++p) {
+    const int pk = p * 64 * W + w * 64 + lane;
+    act[p] = FULL || pk < a.packs;
+    col[p] = pk * kPack;
+    u32x4 r0 = {0, 0, 0, 0};
+    if (act[p]) r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col[p]);
+    unpack8(r0, g[p]);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      comb[wave][0][pi * 8 + j] = acc0[j];
-      if constexpr (ADALN) comb[wave][NACC - 1][pi * 8 + j] = acc1[j];
+      if constexpr (ADALN) g[p][j] += 1.0f;
+      gi[p][j] = (!ADALN && act[p]) ? 1.0f / g[p][j] : 0.f;
+      acc0[p][j] = 0.f;
+      acc1[p][j] = 0.f;
     }
   }
-  __syncthreads();
-  float* base = a.partials + ((size_t)(b * gridDim.x + blockIdx.x) * NACC) * C;
-  for (int i = threadIdx.x; i < NACC * L * 8; i += 64 * NW) {
-    const int acc = i / (L * 8);
-    const int c = i - acc * (L * 8);
-    if (c < C) {
-      float t = comb[0][acc][c];
+
+  u32x4 rawx[R][P], rawd[R][P];
+  float rs[R];
+  auto fetch = [&](int64_t t) {
+    const int64_t r0 = t * (Q * R) + q * R;
 #pragma unroll
-      for (int ww = 1; ww < NW; ++ww) t += comb[ww][acc][c];
-      base[(size_t)acc * C + c] = t;
+    for (int r = 0; r < R; ++r) {
+      const bool ok = r0 + r < S;
+      rs[r] = ok ? a.rstd[b * S + r0 + r] : 0.f;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        rawx[r][p] = u32x4{0, 0, 0, 0};
+        rawd[r][p] = u32x4{0, 0, 0, 0};
+        if (ok && act[p]) {
+          const size_t off = (size_t)((b * S + r0 + r) * C + col[p]);
+          rawx[r][p] = load_stream(a.xs, off);
+          rawd[r][p] = load_stream(a.dy, off);
+        }
+      }
+    }
+  };
+
+  unsigned phase = 0;
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t row0 = tile * (Q * R) + q * R;
+    float xh[R][P][8], df[R][P][8], rstd[R];
+    bool rv[R];
+    if (!PF) fetch(tile);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      rv[r] = row0 + r < S;
+      rstd[r] = rs[r];
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        unpack8(rawx[r][p], xh[r][p]);
+        unpack8(rawd[r][p], df[r][p]);
+      }
+    }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
+
+    float red_v[R * NV];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float s1 = 0.f, s0 = 0.f;
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if constexpr (!ADALN) xh[r][p][j] *= gi[p][j];
+          const float gg = df[r][p][j] * g[p][j];
+          s1 = fmaf(gg, xh[r][p][j], s1);
+          if constexpr (ADALN) s0 += gg;
+        }
+      red_v[r * NV + 0] = s1;
+      if constexpr (ADALN) red_v[r * NV + 1] = s0;
+    }
+    rowgroup_allsum<W, R * NV>(red_v, red[phase & 1][q], w, lane);
+    ++phase;
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat))
+      const float k2 = -rstd[r] * (red_v[r * NV + 0] * a.inv_cols);
+      const float k1 = ADALN ? -rstd[r] * (red_v[r * NV + 1] * a.inv_cols) : 0.f;
+      const int64_t row = b * S + row0 + r;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float dyv = df[r][p][j];
+          acc0[p][j] = fmaf(dyv, xh[r][p][j], acc0[p][j]);
+          if constexpr (ADALN) acc1[p][j] += dyv;
+          o[j] = fmaf(xh[r][p][j], k2, fmaf(dyv * g[p][j], rstd[r], k1));
+        }
+        if (rv[r] && act[p]) store_stream(a.dx, (size_t)(row * C + col[p]), pack8(o));
+      }
     }
   }
+  wide_write_partials<ADALN, W, P, Q>(acc0, acc1, act, col, a.partials, b, C, q, w, lane);
+}
+
+template <int KIND, int L, int R, int NW, bool FULL>
+__global__ __launch_bounds__(64 * NW) void norm_bwd_saved_narrow(const BwdSavedArgs a) {
+  constexpr bool ADALN = (KIND == kAdaLN);
+  constexpr int RPW = 64 / L;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int pi = lane & (L - 1);
+  const int ri = lane / L;
+  const int64_t b = blockIdx.y;
+  const int64_t S = a.rows_per_batch;
+  const int C = a.cols;
+  const bool act = FULL || pi < a.packs;
+  const int col = pi * kPack;
+
+  float g[8], gi[8], acc0[8], acc1[8];
+  {
+    u32x4 r0 = {0, 0, 0, 0};
+    if (act) r0 = load_cached(a.p0, (ADALN ? b * C : 0) + col);
+    unpack8(r0, g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (ADALN) g[j] += 1.0f;
+      gi[j] = (!ADALN && act) ? 1.0f / g[j] : 0.f;
+      acc0[j] = 0.f;
+      acc1[j] = 0.f;
+    }
+  }
+
+  u32x4 rawx[R], rawd[R];
+  float rs[R];
+  auto fetch = [&](int64_t t) {
+    const int64_t rb = t * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t rr = rb + r * RPW;
+      rawx[r] = u32x4{0, 0, 0, 0};
+      rawd[r] = u32x4{0, 0, 0, 0};
+      rs[r] = rr < S ? a.rstd[b * S + rr] : 0.f;
+      if (rr < S && act) {
+        const size_t off = (size_t)((b * S + rr) * C + col);
+        rawx[r] = load_stream(a.xs, off);
+        rawd[r] = load_stream(a.dy, off);
+      }
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  if (PF && tile < a.n_tiles) fetch(tile);
+  for (; tile < a.n_tiles; tile += gridDim.x) {
+    const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
+    float xh[R][8], df[R][8], rstd[R];
+    bool rv[R];
+    if (!PF) fetch(tile);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      rv[r] = rbase + r * RPW < S;
+      rstd[r] = rs[r];
+      unpack8(rawx[r], xh[r]);
+      unpack8(rawd[r], df[r]);
+    }
+    if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float s1 = 0.f, s0 = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if constexpr (!ADALN) xh[r][j] *= gi[j];
+        const float gg = df[r][j] * g[j];
+        s1 = fmaf(gg, xh[r][j], s1);
+        if constexpr (ADALN) s0 += gg;
+      }
+      s1 = group_allsum<L>(s1);
+      if constexpr (ADALN) s0 = group_allsum<L>(s0);
+      const float k2 = -rstd[r] * (s1 * a.inv_cols);
+      const float k1 = ADALN ? -rstd[r] * (s0 * a.inv_cols) : 0.f;
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float dyv = df[r][j];
+        acc0[j] = fmaf(dyv, xh[r][j], acc0[j]);
+        if constexpr (ADALN) acc1[j] += dyv;
+        o[j] = fmaf(xh[r][j], k2, fmaf(dyv * g[j], rstd[r], k1));
+      }
+      if (rv[r] && act) store_stream(a.dx, (size_t)((b * S + rbase + r * RPW) * C + col), pack8(o));
+    }
+  }
+  narrow_write_partials<ADALN, L, NW>(acc0, acc1, a.partials, b, C, pi, ri, wave);
 }
 
 // ============================================================================ second pass
 // out[acc][b][c] = sum_j partials[b][j][acc][c], j in a fixed order: 16 waves take
 // the partials j = wave, wave+16, ... and are then folded in wave order through LDS.
+// The output is fp32, or bf16 (rounded once) when out_bf16 is set.
 template <int NACC>
-__global__ __launch_bounds__(1024) void reduce_partials(float* __restrict__ out0, float* __restrict__ out1,
+__global__ __launch_bounds__(1024) void reduce_partials(void* __restrict__ out0, void* __restrict__ out1,
                                                         const float* __restrict__ partials,
-                                                        int n_partials, int cols) {
+                                                        int n_partials, int cols, int out_bf16) {
   __shared__ float fold[16][NACC][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -664,8 +913,10 @@ __global__ __launch_bounds__(1024) void reduce_partials(float* __restrict__ out0
     float t = fold[0][wave][lane];
 #pragma unroll
     for (int ww = 1; ww < 16; ++ww) t += fold[ww][wave][lane];
-    float* out = wave == 0 ? out0 : out1;
-    out[(size_t)b * cols + c] = t;
+    void* out = wave == 0 ? out0 : out1;
+    const size_t idx = (size_t)b * cols + c;
+    if (out_bf16) static_cast<uint16_t*>(out)[idx] = f32_to_bf16(t);
+    else          static_cast<float*>(out)[idx] = t;
   }
 }
 

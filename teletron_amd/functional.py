@@ -75,12 +75,12 @@ class RMSNormModelFunction(Function):
         return dx, dweight, None, None
 
 
-def fused_adaln(x, shift, scale, eps: float = 1e-6):
+def adaln_modulate(x, shift, scale, eps: float = 1e-6):
     """``modulate(layer_norm(x), shift, scale)`` in one kernel (argument order of ``modulate``)."""
     return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
 
 
-def fused_rmsnorm(x, weight, eps: float = 1e-5):
+def rms_norm(x, weight, eps: float = 1e-5):
     return RMSNormModelFunction.apply(x, weight, eps, x.shape[-1])
 
 

@@ -1,0 +1,121 @@
+"""CPU-side tests: the C-ABI library loads and exports what include/*.h declares, argument
+validation happens before anything touches a GPU, workload bookkeeping is right."""
+import ctypes
+import glob
+import os
+import re
+
+import pytest
+import torch
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for h in glob.glob(os.path.join(REPO, "include", "*.h")):
+        names |= set(re.findall(r"TT_API[^;(]*?\b(tt_[a-z_0-9]+)\s*\(", open(h).read()))
+    return names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = declared_symbols()
+    assert len(names) >= 16
+    for n in sorted(names):
+        assert hasattr(lib, n), f"{n} declared in include/ but not exported"
+    from teletron_amd import cabi
+    assert set(cabi.PROTOTYPES) == names, "ctypes prototypes and header disagree"
+
+
+def test_version_and_error_strings(lib):
+    assert lib.tt_version() >= 100
+    from teletron_amd import cabi
+    texts = {lib.tt_error_string(c) for c in range(0, 6)}
+    assert len(texts) == 6 and b"ok" in texts
+    assert lib.tt_last_hip_error() == 0
+    e = cabi.TeletronOpError("f", 2, "unsupported")
+    assert e.code == 2 and "f failed" in str(e)
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu(lib):
+    from teletron_amd import cabi
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    # null pointers / bad sizes are refused before any HIP call
+    assert lib.tt_rmsnorm_forward(None, p16, p16, None, 4, 64, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_adaln_forward(p16, p16, p16, None, None, None, 4, 64, 4, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_adaln_forward(p16, p16, p16, p16, None, None, 4, 64, 3, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_rmsnorm_forward(p16, p16, p16, None, -1, 64, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_rmsnorm_forward(p16, p16, p16, None, 4, 12, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED      # cols % 8
+    assert lib.tt_rmsnorm_forward(p16, p16, p16, None, 4, 1 << 20, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED  # too wide
+    assert lib.tt_rmsnorm_forward(p16 + 2, p16, p16, None, 4, 64, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED  # misaligned
+    assert lib.tt_launch_rms_forward(p16, p16, p16, 4, 64, 1e-6, None, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_reduce_partials(p16, None, p16, 1, 4, 2, 64, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    # zero rows is a successful no-op
+    assert lib.tt_rmsnorm_forward(None, None, None, None, 0, 64, 1e-6, None) == cabi.TT_OK
+    assert lib.tt_adaln_backward(None, None, None, None, None, None, None, 0, 0, 64, 1, 1e-6, None) == cabi.TT_OK
+    with pytest.raises(cabi.TeletronOpError):
+        cabi.call("tt_rmsnorm_forward", None, p16, p16, None, 4, 64, 1e-6, None)
+
+
+def test_python_validation_on_cpu_tensors():
+    from teletron_amd import AdaLNModelFunction, FusedRMSNorm, RMSNormModelFunction, ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    w = torch.ones(64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.rmsnorm_forward(x, w, 1e-6)
+    with pytest.raises(ValueError, match="not divisible"):
+        RMSNormModelFunction.apply(x, w, 1e-6, 48)
+    with pytest.raises(ValueError, match="not divisible"):
+        AdaLNModelFunction.apply(x, w, w, 1e-6, 60)
+    m = FusedRMSNorm(64, eps=1e-6)
+    assert list(m.state_dict()) == ["weight"] and m.weight.shape == (64,) and bool((m.weight == 1).all())
+    with pytest.raises(ValueError):
+        m(x)   # CPU input: refuses rather than falling back
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from teletron_amd import cabi
+    monkeypatch.setattr(cabi, "_lib", None)
+    monkeypatch.setattr(cabi, "LIB_PATH", tmp_path / "libteletron_op.so")
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        cabi.load()
+
+
+def test_workload_table_matches_the_benchmark_configs():
+    from teletron_amd.workloads import WORKLOADS, make_inputs
+    a = WORKLOADS["adaln_wan14b"]
+    assert (a.rows, a.cols, a.elements) == (75600, 5120, 387072000)
+    assert a.algorithmic_bytes("fwd") == 4 * a.elements + 2 * 5120 * 2
+    assert a.algorithmic_bytes("bwd") == 6 * a.elements + 5120 * 2 + 2 * 5120 * 4
+    h = WORKLOADS["rmsnorm_hunyuan_head"]
+    assert (h.rows, h.cols) == (118800 * 24, 128)
+    assert WORKLOADS["adaln_wan1p3b_batched"].param_shape == (4, 1, 1536)
+    t1 = make_inputs(WORKLOADS["rmsnorm_small"], seed=0, rows=8)
+    t2 = make_inputs(WORKLOADS["rmsnorm_small"], seed=0, rows=8)
+    assert t1["x"].shape == (2, 8, 1536) and t1["x"].dtype == torch.bfloat16
+    assert all(torch.equal(t1[k], t2[k]) for k in t1)
+    assert abs(float(t1["gamma"].float().mean()) - 1.0) < 0.02
+    t3 = make_inputs(WORKLOADS["adaln_odd"], seed=0, rows=4)
+    assert t3["scale"].shape == (3, 1, 1000) and float(t3["scale"].float().std()) < 0.15
+
+
+def test_glue_modules_import_and_register_ops():
+    from teletron_amd import fused_adaln, fused_rmsnorm
+    for mod, names in [(fused_adaln, ["torch_launch_adaln_forward", "torch_launch_adaln_backward"]),
+                       (fused_rmsnorm, ["torch_launch_rms_forward", "torch_launch_rms_backward"])]:
+        for n in names:
+            assert callable(getattr(mod, n))
+    assert torch.ops.layernorm_block_smem.torch_launch_adaln_backward is not None
+    assert torch.ops.Fused_RMSNorm.torch_launch_rms_forward is not None
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        fused_rmsnorm.torch_launch_rms_forward(x, x, torch.ones(64, dtype=torch.bfloat16), 4, 64, 1e-6, torch.zeros(4))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    p = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert p.returncode != 0 and "one GPU" in p.stderr

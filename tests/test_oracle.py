@@ -201,6 +201,25 @@ def test_rmsnorm_special_cases_and_invariants():
     torch.testing.assert_close(dgamma, (dy * x_hat).sum(0), rtol=1e-12, atol=1e-12)
 
 
+def test_saved_tensor_backward_equals_backward_from_x():
+    # Fed the exact x_hat / y and rstd, the reference-contract formulas must reproduce the
+    # gradients already pinned above (which take x).
+    nb, s, c, eps = 1, 9, 40, 1e-6
+    x, sc, sh, dy = rnd(nb, s, c, seed=40, offset=0.5), rnd(1, c, seed=41, scale=0.2), rnd(1, c, seed=42), rnd(nb, s, c, seed=43)
+    _, x_hat, _, rstd = O.adaln_forward(x, sc, sh, eps, 1)
+    dx, dscale, dshift = O.adaln_backward(dy, x, sc, eps, 1)
+    dx2, dscale2, dshift2 = O.adaln_backward_from_saved(dy, x_hat, sc, rstd)
+    torch.testing.assert_close(dx2, dx, rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(dscale2, dscale[0], rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(dshift2, dshift[0], rtol=1e-11, atol=1e-12)
+    gamma = 1 + rnd(c, seed=44, scale=0.2)
+    y, _, rstd = O.rmsnorm_forward(x, gamma, eps)
+    dx, dgamma = O.rmsnorm_backward(dy, x, gamma, eps)
+    dx2, dgamma2 = O.rmsnorm_backward_from_saved(dy, y, gamma, rstd)
+    torch.testing.assert_close(dx2, dx, rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(dgamma2, dgamma, rtol=1e-11, atol=1e-12)
+
+
 def test_chunked_param_grads_match_unchunked():
     nb, s, c, eps = 2, 37, 24, 1e-6
     x, sc, dy = rnd(nb, s, c, seed=27).bfloat16(), rnd(nb, c, seed=28, scale=0.1), rnd(nb, s, c, seed=29).bfloat16()
