@@ -129,19 +129,28 @@ class GpuWorkload:
             torch.cuda.synchronize()
         for i in range(warmup):
             self.fwd(i); self.bwd_partials(i); self.reduce()
-        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(steps):
-            e = ev[i]
-            e[0].record(); self.fwd(i)
-            e[1].record(); self.bwd_partials(i)
-            e[2].record(); self.reduce()
-            e[3].record()
+            self.fwd(i)
+            ev[i][0].record(); self.bwd_partials(i); ev[i][1].record()   # the dominant kernel, timed live
+            self.reduce()
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) / steps
-        us = lambda a, b: [e[a].elapsed_time(e[b]) * 1e3 for e in ev]
-        return wall, {"fwd": us(0, 1), "bwd": us(1, 2), "reduce": us(2, 3)}
+        bwd_us = [e[0].elapsed_time(e[1]) * 1e3 for e in ev]
+        # The two smaller launches are timed in an untimed pass of their own (same buffers, same
+        # order), to keep event packets out of the timed region.
+        n = max(5, min(steps, 20))
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n)]
+        for i in range(n):
+            e = ev[i]
+            e[0].record(); self.fwd(i); e[1].record()
+            self.bwd_partials(i)
+            e[2].record(); self.reduce(); e[3].record()
+        torch.cuda.synchronize()
+        return wall, {"fwd": [e[0].elapsed_time(e[1]) * 1e3 for e in ev], "bwd": bwd_us,
+                      "reduce": [e[2].elapsed_time(e[3]) * 1e3 for e in ev]}
 
 
 def cpu_baseline(w, seconds):
