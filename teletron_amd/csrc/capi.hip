@@ -61,6 +61,7 @@ int resident_wgs_per_cu(const KernelInfo& k, int* out) {
 }
 
 std::atomic<int> g_wgs_per_cu_override{0};
+std::atomic<int> g_grid_override{0};
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -76,7 +77,6 @@ enum Dir { kFwd, kBwd, kBwdSaved };
 
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
 constexpr int kMaxWgsPerCu = 8;
-constexpr int kTargetLoadsPerCu = 18;
 
 int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan) {
   if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0)
@@ -103,16 +103,20 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   if (rc != TT_OK) return rc;
   rc = resident_wgs_per_cu(k, &per_cu);
   if (rc != TT_OK) return rc;
-  // HBM streams fastest with a modest number of requests in flight: measured on
-  // MI355X, throughput peaks near 18 outstanding 128-bit loads per lane-column of
-  // a CU (waves x loads per lane) per streamed tensor and falls off by 10-20 %
-  // at full occupancy.  Tensors that fit the caches just take the whole machine.
+  // HBM streams fastest with a modest number of requests in flight: measured on MI355X,
+  // throughput peaks near kFwdLoadsPerCu / kBwdLoadsPerCu outstanding 128-bit loads per lane
+  // column of a CU (waves x loads per lane) and streamed tensor, falls off by 10-20 % at full
+  // occupancy, and is a few percent better with one CU in 32 left without a workgroup.
+  // Tensors that fit the caches just take the whole machine.
   const bool cache_resident = rows * cols * 2 < (int64_t)64 << 20;
+  int usable_cus = cus;
   if (!cache_resident) {
     const int per_wg = (k.threads / kWave) * k.lane_loads;
-    int want = (kTargetLoadsPerCu + per_wg / 2) / per_wg;
+    const int target = dir == kFwd ? kFwdLoadsPerCu : kBwdLoadsPerCu;
+    int want = (2 * target + per_wg) / (2 * per_wg);
     if (want < 1) want = 1;
     if (want < per_cu) per_cu = want;
+    if (cus >= 32) usable_cus = cus - cus / 32;
   }
   const int ov = g_wgs_per_cu_override.load(std::memory_order_relaxed);
   if (ov > 0) per_cu = ov;
@@ -123,8 +127,10 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   plan->n_batches = rows / rows_per_batch;
   plan->n_tiles = (rows_per_batch + k.tile_rows - 1) / k.tile_rows;
   if (plan->n_batches > 65535) return TT_ERR_UNSUPPORTED;
-  int64_t gx = (int64_t)per_cu * cus / plan->n_batches;
+  int64_t gx = (int64_t)per_cu * usable_cus / plan->n_batches;
   if (gx < 1) gx = 1;
+  const int gov = g_grid_override.load(std::memory_order_relaxed);
+  if (gov > 0 && gov <= kMaxWgsPerCu * cus) gx = gov / plan->n_batches > 0 ? gov / plan->n_batches : 1;
   if (gx > plan->n_tiles) gx = plan->n_tiles;
   plan->grid_x = static_cast<int>(gx);
   return TT_OK;
@@ -254,6 +260,8 @@ int tt_last_hip_error(void) { return g_last_hip_error; }
 // Tuning hook (not part of the public header): force the number of resident
 // workgroups per CU that launch plans assume; 0 restores the occupancy query.
 TT_API void tt_debug_set_wgs_per_cu(int n) { g_wgs_per_cu_override.store(n < 0 ? 0 : n); }
+// Tuning hook: force the total number of workgroups of a launch (0 = off).
+TT_API void tt_debug_set_grid(int n) { g_grid_override.store(n < 0 ? 0 : n); }
 
 int tt_adaln_forward(void* y, const void* x, const void* scale, const void* shift, float* mean, float* rstd,
                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {

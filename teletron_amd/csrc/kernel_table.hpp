@@ -30,18 +30,16 @@ constexpr int kNarrowL[kNumNarrow] = {1, 2, 4, 8, 16, 32};
 constexpr int kNarrowMaxPacks = 32;
 constexpr int kMaxPacks = 64 * 16 * 4;
 
-// ---- tuning constants (rows in flight per row group, row groups per workgroup)
+// ---- tuning constants, from sweeps on MI355X (see make_plan in capi.hip for the grid rule)
+// R: rows in flight per row group;  Q: row groups per workgroup.  HBM throughput peaks with
+// roughly 20 (forward) / 12 (backward, two input tensors) outstanding 128-bit loads per lane
+// column of a CU and tensor, and barrier-coupled row groups in ONE workgroup per CU stream
+// better than independent workgroups; Q is chosen so that one workgroup carries that load.
 #ifndef TT_FWD_R
 #define TT_FWD_R 1
 #endif
-#ifndef TT_FWD_Q
-#define TT_FWD_Q 1
-#endif
 #ifndef TT_BWD_R
 #define TT_BWD_R 1
-#endif
-#ifndef TT_BWD_Q
-#define TT_BWD_Q 1
 #endif
 #ifndef TT_NARROW_FWD_R
 #define TT_NARROW_FWD_R 4
@@ -52,12 +50,29 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 #ifndef TT_NARROW_NW
 #define TT_NARROW_NW 4
 #endif
+constexpr int kFwdLoadsPerCu = 20;   // target waves x loads-per-lane per CU, forward
+constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
 
-constexpr int clampQ(int q, int W) { return (q * W > 16) ? (16 / W > 0 ? 16 / W : 1) : q; }
 constexpr int fwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_FWD_R; }
-constexpr int fwd_wide_Q(int W, int P) { return clampQ(TT_FWD_Q, W); }
 constexpr int bwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_BWD_R; }
-constexpr int bwd_wide_Q(int W, int P) { return clampQ(TT_BWD_Q, W); }
+constexpr int fwd_wide_Q(int W, int P) {
+#ifdef TT_FWD_Q
+  return TT_FWD_Q * W > 16 ? 1 : TT_FWD_Q;
+#else
+  return W >= 7 ? 1 : (10 + W / 2) / W;          // about 10 waves per workgroup
+#endif
+}
+constexpr int bwd_wide_Q(int W, int P) {
+#ifdef TT_BWD_Q
+  return TT_BWD_Q * W > 16 ? 1 : TT_BWD_Q;
+#else
+  int q = (2 * kBwdLoadsPerCu + W * P) / (2 * W * P);   // round(12 / (W*P))
+  if (q < 1) q = 1;
+  if (W * q < 6) q = (6 + W - 1) / W;                   // at least 6 waves to keep up with the arithmetic
+  while (q > 1 && W * q > 12) --q;                      // at most 12 waves: 170 VGPRs per lane
+  return q;
+#endif
+}
 
 // Index of the wide variant for `packs` (> kNarrowMaxPacks), or -1.
 inline int select_wide(int packs) {
