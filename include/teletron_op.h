@@ -7,6 +7,12 @@
  * contiguous: `rows x cols` bf16 for activations, bf16 for parameters, fp32 for
  * per-row statistics and for parameter gradients.
  *
+ * Fast path: cols % 8 == 0 and every tensor 16-byte aligned (128-bit vector kernels).
+ * tt_adaln_forward/backward, tt_rmsnorm_forward/backward and the tt_launch_*_forward entry
+ * points also accept any other cols <= TT_MAX_COLS and 2-byte aligned tensors through
+ * element-wise kernels (a correctness path, several times slower); the two-step backward
+ * and the tt_launch_*_backward entry points return TT_ERR_UNSUPPORTED there.
+ *
  * Two groups of entry points:
  *
  *  1. The native contract (tt_adaln_*, tt_rmsnorm_*): backward consumes the
@@ -42,7 +48,7 @@ extern "C" {
 
 #define TT_OK 0
 #define TT_ERR_INVALID_ARGUMENT 1  /* null pointer, non-positive size, rows % rows_per_batch != 0 */
-#define TT_ERR_UNSUPPORTED 2       /* shape outside what the kernels cover (cols > TT_MAX_COLS) */
+#define TT_ERR_UNSUPPORTED 2       /* shape outside what the entry point covers (see above; cols > TT_MAX_COLS) */
 #define TT_ERR_WORKSPACE 3         /* workspace pointer null or smaller than *_workspace_bytes() */
 #define TT_ERR_HIP 4               /* a HIP runtime call or kernel launch failed */
 
@@ -75,7 +81,9 @@ TT_API int tt_adaln_forward(void* y, const void* x, const void* scale, const voi
  * Inputs dy, x: [rows, cols] bf16; scale: [n_batches, cols] bf16.
  * Outputs dx: [rows, cols] bf16; dscale, dshift: [n_batches, cols] fp32.
  * `workspace` holds the per-workgroup partial column sums; it must be at least
- * tt_adaln_backward_workspace_bytes() and 16-byte aligned.  The result is
+ * tt_adaln_backward_workspace_bytes() and 16-byte aligned.  (With cols % 8 == 0 but a
+ * misaligned tensor the element-wise path needs rows * 8 bytes instead, which can exceed
+ * that figure for very short rows; TT_ERR_WORKSPACE is returned if it does not fit.)  The result is
  * bitwise reproducible run to run (fixed summation order, no atomics).
  */
 TT_API int tt_adaln_backward(void* dx, float* dscale, float* dshift,

@@ -3,9 +3,11 @@
 #include "teletron_op.h"
 
 #include <atomic>
+#include <initializer_list>
 #include <mutex>
 #include <unordered_map>
 
+#include "generic_kernels.hpp"
 #include "kernel_table.hpp"
 
 namespace tt {
@@ -143,6 +145,7 @@ size_t partial_bytes(const Plan& p, int n_acc, int64_t cols) {
 // Workspace bound that does not depend on the launch-time occupancy query.
 size_t workspace_bound(int n_acc, int64_t rows, int64_t cols, int64_t rows_per_batch) {
   if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0) return 0;
+  if (cols % kPack != 0) return (size_t)rows * 2 * sizeof(float);   // element-wise path: row statistics
   int cus = 0;
   if (current_device_cus(&cus) != TT_OK) cus = 256;
   const int64_t n_batches = rows / rows_per_batch;
@@ -161,11 +164,89 @@ int launch(const Plan& p, Args& args, void* stream) {
   return TT_OK;
 }
 
+// ---------------------------------------------------------------- element-wise fallback
+bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+int generic_grid(int64_t rows, int* grid) {
+  int cus = 0;
+  int rc = current_device_cus(&cus);
+  if (rc != TT_OK) return rc;
+  const int64_t cap = (int64_t)cus * 8;
+  *grid = (int)(rows < cap ? rows : cap);
+  return TT_OK;
+}
+
+int check_shape(int64_t rows, int64_t cols, int64_t rows_per_batch) {
+  if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0) return TT_ERR_INVALID_ARGUMENT;
+  if (cols > TT_MAX_COLS || rows / rows_per_batch > 65535) return TT_ERR_UNSUPPORTED;
+  return TT_OK;
+}
+
+int forward_generic(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd,
+                    void* x_norm, int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  int rc = check_shape(rows, cols, rows_per_batch);
+  if (rc != TT_OK) return rc;
+  if (!aligned2(y) || !aligned2(x) || !aligned2(p0) || !aligned2(p1) || !aligned2(x_norm)) return TT_ERR_INVALID_ARGUMENT;
+  int grid = 0;
+  rc = generic_grid(rows, &grid);
+  if (rc != TT_OK) return rc;
+  GenFwdArgs a;
+  a.y = static_cast<uint16_t*>(y); a.x = static_cast<const uint16_t*>(x);
+  a.p0 = static_cast<const uint16_t*>(p0); a.p1 = static_cast<const uint16_t*>(p1);
+  a.mean = mean; a.rstd = rstd; a.x_norm = static_cast<uint16_t*>(x_norm);
+  a.rows = rows; a.rows_per_batch = rows_per_batch; a.cols = (int)cols; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (kind == kAdaLN) hipLaunchKernelGGL(norm_fwd_generic<kAdaLN>, dim3(grid), dim3(kGenThreads), 0, s, a);
+  else                hipLaunchKernelGGL(norm_fwd_generic<kRMS>, dim3(grid), dim3(kGenThreads), 0, s, a);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TT_OK : hip_fail(e);
+}
+
+int backward_generic(int kind, void* dx, void* out0, void* out1, const void* dy, const void* x, const void* p0,
+                     void* workspace, size_t workspace_bytes, int64_t rows, int64_t cols, int64_t rows_per_batch,
+                     float eps, void* stream) {
+  int rc = check_shape(rows, cols, rows_per_batch);
+  if (rc != TT_OK) return rc;
+  if (!dx || !dy || !x || !p0 || !out0 || (kind == kAdaLN && !out1)) return TT_ERR_INVALID_ARGUMENT;
+  if (!aligned2(dx) || !aligned2(dy) || !aligned2(x) || !aligned2(p0)) return TT_ERR_INVALID_ARGUMENT;
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 3u) != 0 ||
+      workspace_bytes < (size_t)rows * 2 * sizeof(float))
+    return TT_ERR_WORKSPACE;
+  int grid = 0;
+  rc = generic_grid(rows, &grid);
+  if (rc != TT_OK) return rc;
+  GenBwdArgs a;
+  a.dx = static_cast<uint16_t*>(dx); a.dy = static_cast<const uint16_t*>(dy); a.x = static_cast<const uint16_t*>(x);
+  a.p0 = static_cast<const uint16_t*>(p0); a.stats = static_cast<float*>(workspace); a.out0 = out0; a.out1 = out1;
+  a.rows = rows; a.rows_per_batch = rows_per_batch; a.cols = (int)cols; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
+  a.out_bf16 = 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 cgrid((unsigned)((cols + 63) / 64), (unsigned)(rows / rows_per_batch), 1);
+  if (kind == kAdaLN) {
+    hipLaunchKernelGGL(norm_bwd_generic<kAdaLN>, dim3(grid), dim3(kGenThreads), 0, s, a);
+    hipLaunchKernelGGL(norm_colgrad_generic<kAdaLN>, cgrid, dim3(1024), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(norm_bwd_generic<kRMS>, dim3(grid), dim3(kGenThreads), 0, s, a);
+    hipLaunchKernelGGL(norm_colgrad_generic<kRMS>, cgrid, dim3(1024), 0, s, a);
+  }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TT_OK : hip_fail(e);
+}
+
+// The vector kernels need 128-bit packs: cols % 8 == 0 and 16-byte aligned tensors.
+bool vector_path(int64_t cols, std::initializer_list<const void*> ptrs) {
+  if (cols % kPack != 0) return false;
+  for (const void* p : ptrs)
+    if (!aligned16(p)) return false;
+  return true;
+}
+
 int forward(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd, void* x_norm,
             int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
   if (rows == 0) return TT_OK;
   if (!y || !x || !p0 || (kind == kAdaLN && !p1)) return TT_ERR_INVALID_ARGUMENT;
-  if (!aligned16(y) || !aligned16(x) || !aligned16(p0) || !aligned16(p1) || !aligned16(x_norm)) return TT_ERR_UNSUPPORTED;
+  if (!vector_path(cols, {y, x, p0, p1, x_norm}))
+    return forward_generic(kind, y, x, p0, p1, mean, rstd, x_norm, rows, cols, rows_per_batch, eps, stream);
   Plan p;
   int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p);
   if (rc != TT_OK) return rc;
@@ -303,6 +384,9 @@ int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, co
                       int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
   if (rows == 0) return TT_OK;
   if (!dscale || !dshift) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {dx, dy, x, scale, workspace}))
+    return backward_generic(kAdaLN, dx, dscale, dshift, dy, x, scale, workspace, workspace_bytes,
+                            rows, cols, rows_per_batch, eps, stream);
   int n_partials = 0;
   int rc = backward_partials(kAdaLN, dx, dy, x, scale, workspace, workspace_bytes, &n_partials,
                              rows, cols, rows_per_batch, eps, stream);
@@ -315,6 +399,9 @@ int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x,
                         int64_t rows, int64_t cols, float eps, void* stream) {
   if (rows == 0) return TT_OK;
   if (!dweight) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {dx, dy, x, weight, workspace}))
+    return backward_generic(kRMS, dx, dweight, nullptr, dy, x, weight, workspace, workspace_bytes,
+                            rows, cols, rows, eps, stream);
   int n_partials = 0;
   int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
                              rows, cols, rows, eps, stream);

@@ -53,6 +53,15 @@ def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int,
     return rows, nb, (rows // nb if nb else rows)
 
 
+def _workspace(lib_bytes: int, rows: int, *tensors: torch.Tensor) -> torch.Tensor:
+    """Backward workspace; tensors that are not 16-byte aligned take the element-wise kernels,
+    which keep two floats of statistics per row there."""
+    need = lib_bytes
+    if any(t.data_ptr() % 16 for t in tensors):
+        need = max(need, rows * 8)
+    return torch.empty(max(need, 16), dtype=torch.uint8, device=tensors[0].device)
+
+
 def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
@@ -97,10 +106,9 @@ def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: 
     dscale = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
     dshift = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        ws_bytes = cabi.load().tt_adaln_backward_workspace_bytes(rows, cols, rpb)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        ws = _workspace(cabi.load().tt_adaln_backward_workspace_bytes(rows, cols, rpb), rows, x, dy, dx, scale)
         cabi.call("tt_adaln_backward", dx.data_ptr(), dscale.data_ptr(), dshift.data_ptr(),
-                  dy.data_ptr(), x.data_ptr(), scale.data_ptr(), ws.data_ptr(), ws_bytes,
+                  dy.data_ptr(), x.data_ptr(), scale.data_ptr(), ws.data_ptr(), ws.numel(),
                   rows, cols, rpb, float(eps), _stream(x))
     return dx, dscale, dshift
 
@@ -135,8 +143,7 @@ def rmsnorm_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, ep
         return dx, torch.zeros(cols, dtype=torch.float32, device=x.device)
     dweight = torch.empty(cols, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        ws_bytes = cabi.load().tt_rmsnorm_backward_workspace_bytes(rows, cols)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        ws = _workspace(cabi.load().tt_rmsnorm_backward_workspace_bytes(rows, cols), rows, x, dy, dx, weight)
         cabi.call("tt_rmsnorm_backward", dx.data_ptr(), dweight.data_ptr(), dy.data_ptr(), x.data_ptr(),
-                  weight.data_ptr(), ws.data_ptr(), ws_bytes, rows, cols, float(eps), _stream(x))
+                  weight.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, float(eps), _stream(x))
     return dx, dweight

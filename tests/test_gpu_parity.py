@@ -145,6 +145,42 @@ def test_rmsnorm_shapes(cols, rows):
     check_rmsnorm(x, gamma, dy, 1e-6, f"rmsnorm[{rows},{cols}]")
 
 
+# ------------------------------------------------------------------ element-wise path: odd widths, misaligned tensors
+@pytest.mark.parametrize("cols", [1, 3, 7, 12, 100, 257, 1001, 5121])
+def test_widths_not_multiple_of_8(cols):
+    x = rand_bf16(2, 37, cols, seed=cols, offset=0.25)
+    if cols == 1:   # a single column normalises to 0: keep the comparison away from 0/0 noise
+        x = x.abs() + 1
+    check_adaln(x, rand_bf16(2, 1, cols, seed=cols + 1, scale=0.1), rand_bf16(2, 1, cols, seed=cols + 2, scale=0.1),
+                rand_bf16(2, 37, cols, seed=cols + 3), 1e-6, 2, f"adaln odd width {cols}")
+    check_rmsnorm(rand_bf16(53, cols, seed=cols + 4), rand_bf16(cols, seed=cols + 5, scale=0.1, offset=1.0),
+                  rand_bf16(53, cols, seed=cols + 6), 1e-6, f"rmsnorm odd width {cols}")
+
+
+def test_misaligned_tensors_take_the_elementwise_path():
+    from teletron_amd import ops
+    rows, cols = 129, 1024
+    base = rand_bf16(rows * cols + 8, seed=50).to(DEV)
+    x = base[4:4 + rows * cols].view(rows, cols)          # 8-byte offset: not 16-byte aligned
+    assert x.is_contiguous() and x.data_ptr() % 16 == 8
+    w = rand_bf16(cols, seed=51, scale=0.1, offset=1.0).to(DEV)
+    dy = rand_bf16(rows, cols, seed=52).to(DEV)
+    y = ops.rmsnorm_forward(x, w, 1e-6)
+    dx, dw = ops.rmsnorm_backward(dy, x, w, 1e-6)
+    xa = x.clone()                                          # same values, aligned: vector kernels
+    y2 = ops.rmsnorm_forward(xa, w, 1e-6)
+    dx2, dw2 = ops.rmsnorm_backward(dy, xa, w, 1e-6)
+    yo, _, _ = O.rmsnorm_forward(x.cpu(), w.cpu(), 1e-6)
+    dxo, dwo = O.rmsnorm_backward(dy.cpu(), x.cpu(), w.cpu(), 1e-6)
+    assert_bf16_close(y, yo, "misaligned y")
+    assert_bf16_close(dx, dxo, "misaligned dx")
+    assert_grad_close(dw, dwo, rows, "misaligned dweight")
+    # both paths round the same fp32 formula: they agree to within one bf16 ulp
+    torch.testing.assert_close(y.float(), y2.float(), rtol=8e-3, atol=1e-3)
+    torch.testing.assert_close(dx.float(), dx2.float(), rtol=8e-3, atol=2e-3)
+    torch.testing.assert_close(dw, dw2, rtol=1e-3, atol=1e-3)
+
+
 def test_many_rows_narrow_and_wide():
     # enough rows that every workgroup of the persistent grid loops several times
     x = rand_bf16(40000, 128, seed=1, scale=1.0)
@@ -265,8 +301,8 @@ def test_argument_errors():
         ops.adaln_forward(x, torch.zeros(3, 64, dtype=torch.bfloat16, device=DEV),
                           torch.zeros(3, 64, dtype=torch.bfloat16, device=DEV), 1e-6)  # 3 does not divide 4 rows
     with pytest.raises(cabi.TeletronOpError) as ei:
-        ops.rmsnorm_forward(torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV),
-                            torch.ones(12, dtype=torch.bfloat16, device=DEV), 1e-6)   # cols % 8 != 0
+        ops.rmsnorm_forward(torch.zeros(4, 40000, dtype=torch.bfloat16, device=DEV),
+                            torch.ones(40000, dtype=torch.bfloat16, device=DEV), 1e-6)   # wider than TT_MAX_COLS
     assert ei.value.code == cabi.TT_ERR_UNSUPPORTED
     # empty input is a no-op
     e = torch.zeros(0, 64, dtype=torch.bfloat16, device=DEV)

@@ -47,9 +47,11 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.tt_adaln_forward(p16, p16, p16, None, None, None, 4, 64, 4, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
     assert lib.tt_adaln_forward(p16, p16, p16, p16, None, None, 4, 64, 3, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
     assert lib.tt_rmsnorm_forward(p16, p16, p16, None, -1, 64, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT
-    assert lib.tt_rmsnorm_forward(p16, p16, p16, None, 4, 12, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED      # cols % 8
     assert lib.tt_rmsnorm_forward(p16, p16, p16, None, 4, 1 << 20, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED  # too wide
-    assert lib.tt_rmsnorm_forward(p16 + 2, p16, p16, None, 4, 64, 1e-6, None) == cabi.TT_ERR_UNSUPPORTED  # misaligned
+    assert lib.tt_rmsnorm_forward(p16 + 1, p16, p16, None, 4, 64, 1e-6, None) == cabi.TT_ERR_INVALID_ARGUMENT  # odd address
+    n = ctypes.c_int(-1)
+    assert lib.tt_rmsnorm_backward_partials(p16, p16, p16, p16, p16, 64, ctypes.byref(n), 4, 12, 1e-6, None) \
+        == cabi.TT_ERR_UNSUPPORTED and n.value == 0                                                         # cols % 8, two-step API
     assert lib.tt_launch_rms_forward(p16, p16, p16, 4, 64, 1e-6, None, None) == cabi.TT_ERR_INVALID_ARGUMENT
     assert lib.tt_reduce_partials(p16, None, p16, 1, 4, 2, 64, None) == cabi.TT_ERR_INVALID_ARGUMENT
     # zero rows is a successful no-op
