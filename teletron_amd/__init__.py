@@ -5,10 +5,10 @@ The compute path is hand-written HIP for gfx950 in ``libteletron_op.so`` (C ABI,
 """
 from .functional import (AdaLNModelFunction, FusedAdaLN, FusedRMSNorm, RMSNormModelFunction,
                          adaln_modulate, rms_norm)
-from . import cabi, ops, workloads
+from . import cabi, ops, swap_in, workloads
 
 __all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "FusedAdaLN", "FusedRMSNorm",
-           "adaln_modulate", "rms_norm", "cabi", "ops", "workloads", "install_reference_modules"]
+           "adaln_modulate", "rms_norm", "cabi", "ops", "swap_in", "workloads", "install_reference_modules"]
 
 
 def install_reference_modules() -> None:

@@ -1,0 +1,162 @@
+"""Swap the fused kernels into TeleTron model code without editing it.
+
+TeleTron gates its fused ops behind ``FUSED_KERNELS=1`` (``teletron_op/README.md:6``) but
+ships no code that performs the swap.  This module does it by patching *instances*:
+
+* every ``RMSNorm``-style module (``weight`` + ``eps`` + ``norm`` method, as in
+  ``teletron/models/wan/wan_model.py:113-124``) gets a fused ``forward``; parameters and
+  state-dict keys are untouched;
+* every ``nn.LayerNorm(dim, eps, elementwise_affine=False)`` that feeds a modulation
+  (``norm1`` / ``norm2`` of ``DiTBlock`` and ``ContextParallelWanDitBlock``, ``norm`` of
+  ``Head`` and of the HunyuanVideo ``AdaLayerNormZero[Single]``:
+  ``wan_model.py:222-223,236,241,271,277``, ``parallel_wan_model.py:23-24,32-33``,
+  ``hunyuan/model.py:444,467,484,502``) is replaced by :class:`DeferredLayerNorm`.  It does not
+  normalise; it hands back a :class:`DeferredNorm` token that the *consumer* turns into one
+  fused AdaLN launch:
+    - ``modulate(token, shift, scale)``: the module-level function of the Wan model file or the
+      ``modulate`` / ``modulate_with_cp_grad_reduce`` attribute of the block, wrapped by
+      :func:`fused_modulate`;
+    - ``token * (1 + scale) + shift`` written inline (``wan_model.py:277``): the token's
+      ``__mul__`` / ``__add__`` do the same.
+  Anything else done to a token raises, so a missed consumer cannot silently compute garbage.
+
+Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` all-reduces dscale/dshift over the
+context-parallel group (``core/context_parallel/layers.py:49-52``); with a group of size 1 that is
+the identity, which is what the fused op returns.
+"""
+from __future__ import annotations
+
+import os
+import types
+from typing import Callable, Iterable, Optional
+
+import torch
+import torch.nn as nn
+
+from .functional import AdaLNModelFunction, RMSNormModelFunction
+
+ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
+ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
+MODULATE_ATTRS = ("modulate", "modulate_with_cp_grad_reduce")
+
+
+def fused_kernels_requested() -> bool:
+    """The reference's switch: environment variable FUSED_KERNELS=1."""
+    return os.environ.get("FUSED_KERNELS", "0") == "1"
+
+
+class DeferredNorm:
+    """Token for 'LayerNorm(x) not computed yet'.  Holds x and eps until the modulation arrives."""
+
+    __slots__ = ("x", "eps", "one_plus_scale")
+
+    def __init__(self, x: torch.Tensor, eps: float, one_plus_scale: Optional[torch.Tensor] = None):
+        self.x, self.eps, self.one_plus_scale = x, eps, one_plus_scale
+
+    # inline form:  token * (1 + scale) + shift
+    def __mul__(self, one_plus_scale):
+        if self.one_plus_scale is not None or not isinstance(one_plus_scale, torch.Tensor):
+            raise TypeError("DeferredNorm supports exactly `norm(x) * (1 + scale) + shift`")
+        return DeferredNorm(self.x, self.eps, one_plus_scale)
+
+    __rmul__ = __mul__
+
+    def __add__(self, shift):
+        if self.one_plus_scale is None or not isinstance(shift, torch.Tensor):
+            raise TypeError("DeferredNorm supports exactly `norm(x) * (1 + scale) + shift`")
+        # (1 + scale) was rounded to the activation dtype by the caller; subtracting 1 is exact
+        # there, so the kernel multiplies by the very factor the eager expression would use.
+        return modulate_token(self, shift, self.one_plus_scale - 1)
+
+    __radd__ = __add__
+
+    def materialize(self) -> torch.Tensor:
+        """Plain LayerNorm, for a consumer that is not a modulation."""
+        return torch.nn.functional.layer_norm(self.x, (self.x.shape[-1],), eps=self.eps)
+
+    def __getattr__(self, name):
+        raise AttributeError(
+            f"DeferredNorm has no attribute {name!r}: the output of a swapped LayerNorm may only be passed to "
+            "`modulate(...)` or used as `norm(x) * (1 + scale) + shift`; call .materialize() for anything else")
+
+
+def modulate_token(token: DeferredNorm, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    x = token.x
+    return AdaLNModelFunction.apply(x, scale, shift, token.eps, x.shape[-1])
+
+
+def fused_modulate(original: Callable) -> Callable:
+    """Wrap a ``modulate(x, shift, scale)`` callable: tokens take the fused kernel, tensors the original."""
+
+    def modulate(x, shift, scale):
+        if isinstance(x, DeferredNorm):
+            return modulate_token(x, shift, scale)
+        return original(x, shift, scale)
+
+    modulate.__wrapped__ = original
+    return modulate
+
+
+class DeferredLayerNorm(nn.Module):
+    """Stands in for ``nn.LayerNorm(dim, eps, elementwise_affine=False)``; parameter-free, so
+    replacing the original changes no state-dict key."""
+
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.normalized_shape, self.eps = (dim,), eps
+
+    def forward(self, x: torch.Tensor):
+        if x.is_cuda and x.dtype == torch.bfloat16:
+            return DeferredNorm(x, self.eps)
+        return torch.nn.functional.layer_norm(x, self.normalized_shape, eps=self.eps)
+
+    def extra_repr(self) -> str:
+        return f"{self.normalized_shape}, eps={self.eps}, fused with the following modulation"
+
+
+def _is_rmsnorm(m: nn.Module) -> bool:
+    return (type(m).__name__ == "RMSNorm" and isinstance(getattr(m, "weight", None), nn.Parameter)
+            and m.weight.dim() == 1 and hasattr(m, "eps"))
+
+
+def _fused_rmsnorm_forward(self, x: torch.Tensor) -> torch.Tensor:
+    if x.is_cuda and x.dtype == torch.bfloat16:
+        return RMSNormModelFunction.apply(x, self.weight, self.eps, x.shape[-1])
+    return type(self).forward(self, x)
+
+
+def _is_plain_layernorm(m) -> bool:
+    return (isinstance(m, nn.LayerNorm) and not m.elementwise_affine and len(m.normalized_shape) == 1)
+
+
+def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool = True, adaln: bool = True) -> dict:
+    """Patch ``model`` in place.  ``namespaces`` are Python modules (e.g. the imported
+    ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
+    tokens.  Returns counts of what was swapped."""
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0}
+    for ns in namespaces:
+        fn = getattr(ns, "modulate", None)
+        if callable(fn) and not hasattr(fn, "__wrapped__"):
+            setattr(ns, "modulate", fused_modulate(fn))
+            counts["modulate"] += 1
+    for module in list(model.modules()):
+        if rmsnorm and _is_rmsnorm(module) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(_fused_rmsnorm_forward, module)
+            counts["rmsnorm"] += 1
+        if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
+            for attr in MODULATE_ATTRS:
+                fn = getattr(module, attr, None)
+                if callable(fn) and not hasattr(fn, "__wrapped__"):
+                    setattr(module, attr, fused_modulate(fn))
+                    counts["modulate"] += 1
+            for attr in ADALN_NORM_ATTRS:
+                ln = getattr(module, attr, None)
+                if _is_plain_layernorm(ln):
+                    setattr(module, attr, DeferredLayerNorm(ln.normalized_shape[0], ln.eps))
+                    counts["layernorm"] += 1
+    return counts
+
+
+def swap_in_if_requested(model: nn.Module, namespaces: Iterable[object] = ()) -> Optional[dict]:
+    """``swap_in`` when FUSED_KERNELS=1, else leave the model alone."""
+    return swap_in(model, namespaces) if fused_kernels_requested() else None
