@@ -137,6 +137,25 @@ TT_API int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x,
 TT_API int tt_reduce_partials(float* out0, float* out1, const void* workspace,
                        int n_batches, int n_partials, int n_acc, int64_t cols, void* stream);
 
+/* ------------------------------------------------------------------ gated residual add
+ * out = x + gate * residual, the op that follows each fused AdaLN site in a DiT block;
+ * gate is [n_batches, cols] bf16, broadcast over the rows of its batch.  teletron_op has no
+ * kernel for it: the reference runs it as eager torch ops in GateModule.forward
+ * (teletron/models/wan/wan_model.py:205-210) / GateWithGradReduce
+ * (teletron/core/context_parallel/layers.py:24-36), whose arithmetic this replaces:
+ *   forward   out = x + gate * residual
+ *   backward  dresidual = dout * gate;  dgate[b, c] = sum_{rows of batch b} dout * residual
+ *             (dx = dout: no kernel, the caller aliases it)
+ * Vector path only (cols % 8 == 0, 16-byte aligned tensors).  dgate is fp32 [n_batches, cols],
+ * reduced in a fixed order like the other parameter gradients.
+ */
+TT_API int tt_gate_residual_forward(void* out, const void* x, const void* gate, const void* residual,
+                                    int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream);
+TT_API int tt_gate_residual_backward(void* dresidual, float* dgate, const void* dout, const void* gate,
+                                     const void* residual, void* workspace, size_t workspace_bytes,
+                                     int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream);
+TT_API size_t tt_gate_residual_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch);
+
 /* ------------------------------------------------------------------ reference-compatible contract
  * Argument for argument the launchers the reference's pybind glue calls, plus a trailing
  * stream (the reference launches on the legacy default stream) and, for backward, the

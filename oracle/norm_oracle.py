@@ -174,6 +174,24 @@ def rmsnorm_backward_from_saved(dy, y, gamma, rstd):
     return dx.reshape(y.shape), (dyf * xh).sum(dim=0)
 
 
+# --------------------------------------------------------------------------- gated residual add
+def gate_residual_forward(x, gate, residual, n_batches: int = 1):
+    """out = x + gate * residual (teletron/models/wan/wan_model.py:205-210); gate [B, C]."""
+    c = x.shape[-1]
+    g = _param(gate, n_batches, c)[:, None, :]
+    return (_bsc(x, n_batches) + g * _bsc(residual, n_batches)).reshape(x.shape)
+
+
+def gate_residual_backward(dout, gate, residual, n_batches: int = 1):
+    """(dx, dgate[B,C], dresidual) of the above, as written out by hand in
+    teletron/core/context_parallel/layers.py:31-36: dx = dout, dresidual = dout * gate,
+    dgate = sum over the rows of a batch of dout * residual."""
+    c = dout.shape[-1]
+    d, r = _bsc(dout, n_batches), _bsc(residual, n_batches)
+    g = _param(gate, n_batches, c)[:, None, :]
+    return _f64(dout), (d * r).sum(dim=1), (d * g).reshape(dout.shape)
+
+
 # --------------------------------------------------------------------------- chunked variants
 def adaln_backward_param_grads_chunked(dy, x, eps: float, n_batches: int = 1, chunk_rows: int = 4096):
     """dscale / dshift only, streamed over row chunks so that full-size shapes

@@ -3,11 +3,11 @@
 The compute path is hand-written HIP for gfx950 in ``libteletron_op.so`` (C ABI,
 ``include/teletron_op.h``); Python only validates, allocates and launches.
 """
-from .functional import (AdaLNModelFunction, FusedAdaLN, FusedRMSNorm, RMSNormModelFunction,
-                         adaln_modulate, rms_norm)
+from .functional import (AdaLNModelFunction, FusedAdaLN, FusedGate, FusedRMSNorm, GateResidualFunction,
+                         RMSNormModelFunction, adaln_modulate, rms_norm)
 from . import cabi, ops, swap_in, workloads
 
-__all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "FusedAdaLN", "FusedRMSNorm",
+__all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "GateResidualFunction", "FusedAdaLN", "FusedRMSNorm", "FusedGate",
            "adaln_modulate", "rms_norm", "cabi", "ops", "swap_in", "workloads", "install_reference_modules"]
 
 

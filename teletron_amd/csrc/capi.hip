@@ -76,6 +76,7 @@ struct Plan {
 };
 
 enum Dir { kFwd, kBwd, kBwdSaved };
+constexpr int kGateKind = 2;   // third op family next to kAdaLN / kRMS
 
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
 constexpr int kMaxWgsPerCu = 8;
@@ -95,9 +96,11 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   if (kind == kAdaLN)
     k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
-  else
+  else if (kind == kRMS)
     k = dir == kFwd ? rms_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? rms_bwd_kernel(narrow, idx, full) : rms_bwd_saved_kernel(narrow, idx, full);
+  else
+    k = dir == kFwd ? gate_fwd_kernel(narrow, idx, full) : gate_bwd_kernel(narrow, idx, full);
   if (!k.fn) return TT_ERR_UNSUPPORTED;
 
   int cus = 0, per_cu = 0;
@@ -114,7 +117,8 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   int usable_cus = cus;
   if (!cache_resident) {
     const int per_wg = (k.threads / kWave) * k.lane_loads;
-    const int target = dir == kFwd ? kFwdLoadsPerCu : kBwdLoadsPerCu;
+    // two streamed inputs (backward kernels, both gate kernels) or one (normalisation forward)
+    const int target = (dir == kFwd && kind != kGateKind) ? kFwdLoadsPerCu : kBwdLoadsPerCu;
     int want = (2 * target + per_wg) / (2 * per_wg);
     if (want < 1) want = 1;
     if (want < per_cu) per_cu = want;
@@ -407,6 +411,43 @@ int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x,
                              rows, cols, rows, eps, stream);
   if (rc != TT_OK) return rc;
   return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, false, stream);
+}
+
+// ---------------------------------------------------------------- gated residual add
+int tt_gate_residual_forward(void* out, const void* x, const void* gate, const void* residual,
+                             int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!out || !x || !gate || !residual) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {out, x, gate, residual})) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kGateKind, kFwd, rows, cols, rows_per_batch, &p);
+  if (rc != TT_OK) return rc;
+  GateArgs a;
+  a.out = out; a.a = x; a.b = residual; a.gate = gate; a.partials = nullptr;
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles; a.cols = (int)cols; a.packs = p.packs;
+  return launch(p, a, stream);
+}
+
+size_t tt_gate_residual_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch) {
+  return cols % kPack == 0 ? workspace_bound(1, rows, cols, rows_per_batch) : 0;
+}
+
+int tt_gate_residual_backward(void* dresidual, float* dgate, const void* dout, const void* gate,
+                              const void* residual, void* workspace, size_t workspace_bytes,
+                              int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dresidual || !dgate || !dout || !gate || !residual) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {dresidual, dout, gate, residual})) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kGateKind, kBwd, rows, cols, rows_per_batch, &p);
+  if (rc != TT_OK) return rc;
+  if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, 1, cols)) return TT_ERR_WORKSPACE;
+  GateArgs a;
+  a.out = dresidual; a.a = dout; a.b = residual; a.gate = gate; a.partials = static_cast<float*>(workspace);
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles; a.cols = (int)cols; a.packs = p.packs;
+  rc = launch(p, a, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dgate, nullptr, workspace, (int)(rows / rows_per_batch), p.grid_x, 1, cols, false, stream);
 }
 
 // ---------------------------------------------------------------- reference-compatible contract

@@ -3,6 +3,7 @@
 // forward / backward) is instantiated in its own translation unit through the
 // lookup templates below, so the families compile in parallel.
 #pragma once
+#include "gate_kernels.hpp"
 #include "norm_kernels.hpp"
 
 namespace tt {
@@ -156,6 +157,34 @@ KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
+template <int MODE, int W, int P, bool FULL>
+KernelInfo info_gate_wide() {
+  constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&gate_wide<MODE, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
+}
+template <int MODE, int L, bool FULL>
+KernelInfo info_gate_narrow() {
+  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&gate_narrow<MODE, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
+}
+template <int MODE>
+KernelInfo lookup_gate(bool narrow, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L) case i: return full ? info_gate_narrow<MODE, L, true>() : info_gate_narrow<MODE, L, false>();
+      TT_NARROW_LIST(X)
+#undef X
+    }
+  } else {
+    switch (idx) {
+#define X(i, W, P) case i: return full ? info_gate_wide<MODE, W, P, true>() : info_gate_wide<MODE, W, P, false>();
+      TT_WIDE_LIST(X)
+#undef X
+    }
+  }
+  return {nullptr, 0, 0, 0};
+}
+
 template <int KIND>
 KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   if (narrow) {
@@ -174,12 +203,14 @@ KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
-// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip).
+// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, gate.hip).
 KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_saved_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
+KernelInfo gate_fwd_kernel(bool narrow, int idx, bool full);
+KernelInfo gate_bwd_kernel(bool narrow, int idx, bool full);
 
 }  // namespace tt

@@ -75,6 +75,38 @@ class RMSNormModelFunction(Function):
         return dx, dweight, None, None
 
 
+class GateResidualFunction(Function):
+    """``x + gate * residual`` with the hand-written backward of ``GateWithGradReduce``
+    (``teletron/core/context_parallel/layers.py:24-36``) on one GPU: returns
+    ``(dout, sum_rows(dout * residual), dout * gate)``, dgate reduced in fp32."""
+
+    @staticmethod
+    def forward(ctx, x, gate, residual):
+        ctx.gate_meta = (gate.shape, gate.dtype)
+        gate_c = gate.detach().to(torch.bfloat16).contiguous()
+        residual = residual.contiguous()
+        ctx.save_for_backward(gate_c, residual)
+        return ops.gate_residual_forward(x.contiguous(), gate_c, residual)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        gate_c, residual = ctx.saved_tensors
+        g_shape, g_dtype = ctx.gate_meta
+        if not (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]):
+            return grad_output, None, None
+        dres, dgate = ops.gate_residual_backward(grad_output.contiguous(), gate_c, residual)
+        return (grad_output if ctx.needs_input_grad[0] else None,
+                dgate.to(g_dtype).reshape(g_shape) if ctx.needs_input_grad[1] else None,
+                dres if ctx.needs_input_grad[2] else None)
+
+
+class FusedGate(nn.Module):
+    """Drop-in for ``GateModule`` (``teletron/models/wan/wan_model.py:205-210``): ``forward(x, gate, residual)``."""
+
+    def forward(self, x: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        return GateResidualFunction.apply(x, gate, residual)
+
+
 def adaln_modulate(x, shift, scale, eps: float = 1e-6):
     """``modulate(layer_norm(x), shift, scale)`` in one kernel (argument order of ``modulate``)."""
     return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])

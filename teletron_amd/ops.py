@@ -147,3 +147,40 @@ def rmsnorm_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, ep
         cabi.call("tt_rmsnorm_backward", dx.data_ptr(), dweight.data_ptr(), dy.data_ptr(), x.data_ptr(),
                   weight.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, float(eps), _stream(x))
     return dx, dweight
+
+
+def gate_residual_forward(x: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+    """out = x + gate * residual; gate holds n_batches * cols elements (e.g. [B, 1, C])."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    residual = _check_act("residual", residual, cols)
+    _require(residual.numel() == x.numel() and residual.device == x.device, ValueError,
+             "residual must match x in size and device")
+    gate = _check_param("gate", gate, x, cols)
+    rows, nb, rpb = _batches(x, gate, cols)
+    out = torch.empty_like(x)
+    if rows:
+        with torch.cuda.device(x.device):
+            cabi.call("tt_gate_residual_forward", out.data_ptr(), x.data_ptr(), gate.data_ptr(), residual.data_ptr(),
+                      rows, cols, rpb, _stream(x))
+    return out
+
+
+def gate_residual_backward(dout: torch.Tensor, gate: torch.Tensor, residual: torch.Tensor):
+    """Returns (dresidual bf16 like residual, dgate fp32 [n_batches, C]); dx is dout itself."""
+    cols = dout.shape[-1]
+    dout = _check_act("dout", dout, cols)
+    residual = _check_act("residual", residual, cols)
+    _require(residual.numel() == dout.numel() and residual.device == dout.device, ValueError,
+             "residual must match dout in size and device")
+    gate = _check_param("gate", gate, dout, cols)
+    rows, nb, rpb = _batches(dout, gate, cols)
+    dres = torch.empty_like(residual)
+    if rows == 0:
+        return dres, torch.zeros(nb, cols, dtype=torch.float32, device=dout.device)
+    dgate = torch.empty(nb, cols, dtype=torch.float32, device=dout.device)
+    with torch.cuda.device(dout.device):
+        ws = _workspace(cabi.load().tt_gate_residual_backward_workspace_bytes(rows, cols, rpb), 0, dout)
+        cabi.call("tt_gate_residual_backward", dres.data_ptr(), dgate.data_ptr(), dout.data_ptr(), gate.data_ptr(),
+                  residual.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, rpb, _stream(dout))
+    return dres, dgate

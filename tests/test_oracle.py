@@ -220,6 +220,22 @@ def test_saved_tensor_backward_equals_backward_from_x():
     torch.testing.assert_close(dgamma2, dgamma, rtol=1e-11, atol=1e-12)
 
 
+def test_gate_residual_matches_autograd():
+    nb, s, c = 3, 5, 24
+    x, r, dy = rnd(nb, s, c, seed=50).requires_grad_(True), rnd(nb, s, c, seed=51).requires_grad_(True), rnd(nb, s, c, seed=52)
+    g = rnd(nb, 1, c, seed=53, scale=0.5).requires_grad_(True)
+    out = x + g * r
+    out.backward(dy)
+    torch.testing.assert_close(O.gate_residual_forward(x, g, r, nb), out.detach(), rtol=1e-13, atol=1e-13)
+    dx, dgate, dres = O.gate_residual_backward(dy, g, r, nb)
+    torch.testing.assert_close(dx, x.grad, rtol=0, atol=0)
+    torch.testing.assert_close(dgate, g.grad.reshape(nb, c), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(dres, r.grad, rtol=1e-12, atol=1e-12)
+    # gate == 0 passes x through; gate == 1 is a plain residual add
+    torch.testing.assert_close(O.gate_residual_forward(x, torch.zeros(nb, c), r, nb), x.detach(), rtol=0, atol=0)
+    torch.testing.assert_close(O.gate_residual_forward(x, torch.ones(nb, c), r, nb), (x + r).detach(), rtol=0, atol=1e-15)
+
+
 def test_chunked_param_grads_match_unchunked():
     nb, s, c, eps = 2, 37, 24, 1e-6
     x, sc, dy = rnd(nb, s, c, seed=27).bfloat16(), rnd(nb, c, seed=28, scale=0.1), rnd(nb, s, c, seed=29).bfloat16()
