@@ -154,6 +154,7 @@ __global__ __launch_bounds__(64 * NW) void gate_narrow(const GateArgs a) {
       unpack8(rawb[r], bf[r]);
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
+    if constexpr (NW > 1) __syncthreads();   // lock-step only, as in gate_wide
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float o[8];

@@ -33,7 +33,7 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 
 // ---- tuning constants, from sweeps on MI355X (see make_plan in capi.hip for the grid rule)
 // R: rows in flight per row group;  Q: row groups per workgroup.  HBM throughput peaks with
-// roughly 20 (forward) / 12 (backward, two input tensors) outstanding 128-bit loads per lane
+// roughly 18 (forward) / 12 (backward, two input tensors) outstanding 128-bit loads per lane
 // column of a CU and tensor, and barrier-coupled row groups in ONE workgroup per CU stream
 // better than independent workgroups; Q is chosen so that one workgroup carries that load.
 #ifndef TT_FWD_R
@@ -43,7 +43,7 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 #define TT_BWD_R 1
 #endif
 #ifndef TT_NARROW_FWD_R
-#define TT_NARROW_FWD_R 4
+#define TT_NARROW_FWD_R 2
 #endif
 #ifndef TT_NARROW_BWD_R
 #define TT_NARROW_BWD_R 2
@@ -51,7 +51,7 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 #ifndef TT_NARROW_NW
 #define TT_NARROW_NW 4
 #endif
-constexpr int kFwdLoadsPerCu = 20;   // target waves x loads-per-lane per CU, forward
+constexpr int kFwdLoadsPerCu = 18;   // target waves x loads-per-lane per CU, forward
 constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
 
 constexpr int fwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_FWD_R; }

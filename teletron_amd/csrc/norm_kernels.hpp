@@ -611,6 +611,7 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       unpack8(rawd[r], df[r]);
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
+    if constexpr (NW > 1) __syncthreads();   // lock-step only: keeps the request stream narrow (+1-2 %)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float mean = 0.f;
@@ -855,6 +856,7 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_saved_narrow(const BwdSavedA
       unpack8(rawd[r], df[r]);
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
+    if constexpr (NW > 1) __syncthreads();   // lock-step only: keeps the request stream narrow (+1-2 %)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float s1 = 0.f, s0 = 0.f;

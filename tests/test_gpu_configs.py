@@ -138,3 +138,35 @@ def test_rmsnorm_wan14b_qk_full_size():
 
 def test_rmsnorm_hunyuan_head_full_size():
     _rmsnorm_full_size("rmsnorm_hunyuan_head", 1 << 18)
+
+
+def test_more_than_2_31_elements():
+    """Row offsets are 64-bit: a tensor with more than 2^31 elements (the reference's backward
+    kernel keeps `row * cols` in an int, adaln_backward.cu:78) is normalised correctly to its end."""
+    from teletron_amd import ops
+    rows, cols = 540000, 4096                       # 2.21e9 elements, 4.4 GB per tensor
+    assert rows * cols > 2 ** 31
+    g = torch.Generator(device=DEV).manual_seed(3)
+    x = torch.empty(rows, cols, dtype=torch.bfloat16, device=DEV)
+    dy = torch.empty(rows, cols, dtype=torch.bfloat16, device=DEV)
+    for blk in range(0, rows, 60000):               # fill in blocks: no fp32 temporaries of the full size
+        n = min(60000, rows - blk)
+        x[blk:blk + n] = torch.randn(n, cols, generator=g, device=DEV).to(torch.bfloat16)
+        dy[blk:blk + n] = torch.randn(n, cols, generator=g, device=DEV).to(torch.bfloat16)
+    scale = (0.1 * torch.randn(1, cols, generator=g, device=DEV)).to(torch.bfloat16)
+    shift = (0.1 * torch.randn(1, cols, generator=g, device=DEV)).to(torch.bfloat16)
+    y = ops.adaln_forward(x, scale, shift, 1e-6)
+    dx, dscale, dshift = ops.adaln_backward(dy, x, scale, 1e-6)
+    idx = torch.cat([torch.arange(0, 4), torch.arange(rows - 4, rows),
+                     torch.randint(2 ** 31 // cols - 8, rows, (256,), generator=torch.Generator().manual_seed(4))])
+    xs, dys = x[idx.to(DEV)].cpu(), dy[idx.to(DEV)].cpu()
+    yo, _, _, _ = O.adaln_forward(xs, scale.cpu(), shift.cpu(), 1e-6, 1)
+    dxo, _, _ = O.adaln_backward(dys, xs, scale.cpu(), 1e-6, 1)
+    assert_bf16_close(y[idx.to(DEV)], yo, "y beyond 2^31")
+    assert_bf16_close(dx[idx.to(DEV)], dxo, "dx beyond 2^31")
+    # dshift is a plain column sum of dy over every row: a wrapped offset would miss rows
+    ref = torch.zeros(cols, dtype=torch.float64, device=DEV)
+    for blk in range(0, rows, 60000):
+        ref += dy[blk:blk + 60000].double().sum(0)
+    assert_grad_close(dshift, ref.cpu(), rows, "dshift over all rows")
+    assert torch.isfinite(dscale).all()
