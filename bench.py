@@ -63,7 +63,7 @@ class GpuWorkload:
         self.lib = cabi.load()
         dev = torch.device("cuda:0")
         self.rows, self.cols = w.rows, w.cols
-        self.nb = w.param_shape[0] if w.op == "adaln" else 1
+        self.nb = w.param_shape[0] if w.op in ("adaln", "gate") else 1
         self.rpb = self.rows // self.nb
         g = torch.Generator(device=dev).manual_seed(seed)
         bf = torch.bfloat16
@@ -77,7 +77,13 @@ class GpuWorkload:
                  "y": torch.empty(self.rows, self.cols, dtype=bf, device=dev),
                  "dx": torch.empty(self.rows, self.cols, dtype=bf, device=dev)}
             self.sets.append(s)
-        if w.op == "adaln":
+        if w.op == "gate":
+            # x / dy double as (x, residual) forward and (dout, residual) backward
+            self.p0 = randn(self.nb, self.cols, scale=0.5)                 # gate
+            self.p1 = None
+            self.n_acc = 1
+            ws_bytes = self.lib.tt_gate_residual_backward_workspace_bytes(self.rows, self.cols, self.rpb)
+        elif w.op == "adaln":
             self.p0 = randn(self.nb, self.cols, scale=0.1)                 # scale
             self.p1 = randn(self.nb, self.cols, scale=0.1)                 # shift
             self.n_acc = 2
@@ -95,7 +101,10 @@ class GpuWorkload:
 
     def fwd(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "adaln":
+        if self.w.op == "gate":
+            self.cabi.call("tt_gate_residual_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
+                           s["dy"].data_ptr(), self.rows, self.cols, self.rpb, self.stream)
+        elif self.w.op == "adaln":
             self.cabi.call("tt_adaln_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
                            self.p1.data_ptr(), None, None, self.rows, self.cols, self.rpb, self.w.eps, self.stream)
         else:
@@ -104,7 +113,11 @@ class GpuWorkload:
 
     def bwd_partials(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "adaln":
+        if self.w.op == "gate":          # one entry point: streaming kernel + reduction of its partials
+            self.cabi.call("tt_gate_residual_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
+                           self.p0.data_ptr(), s["x"].data_ptr(), self.ws.data_ptr(), self.ws.numel(),
+                           self.rows, self.cols, self.rpb, self.stream)
+        elif self.w.op == "adaln":
             self.cabi.call("tt_adaln_backward_partials", s["dx"].data_ptr(), s["dy"].data_ptr(), s["x"].data_ptr(),
                            self.p0.data_ptr(), self.ws.data_ptr(), self.ws.numel(), ctypes.byref(self.n_partials),
                            self.rows, self.cols, self.rpb, self.w.eps, self.stream)
@@ -114,6 +127,8 @@ class GpuWorkload:
                            self.rows, self.cols, self.w.eps, self.stream)
 
     def reduce(self):
+        if self.w.op == "gate":
+            return
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
 
@@ -162,7 +177,9 @@ def cpu_baseline(w, seconds):
     sample_rows = min(w.shape[1], 16384)
     t = make_inputs(w, seed=0, rows=sample_rows)
     elements = t["x"].numel()
-    if w.op == "adaln":
+    if w.op == "gate":
+        fn = lambda: E.eager_gate_fwd_bwd(t["x"], t["gate"], t["residual"], t["dy"])
+    elif w.op == "adaln":
         fn = lambda: E.eager_adaln_fwd_bwd(t["x"], t["scale"], t["shift"], t["dy"], w.eps)
     else:
         fn = lambda: E.eager_rmsnorm_fwd_bwd(t["x"], t["gamma"], t["dy"], w.eps)
@@ -174,10 +191,11 @@ def cpu_baseline(w, seconds):
         if len(times) >= 2000:
             break
     med = statistics.median(times)
-    return {"value": round(10.0 * elements / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+    per_elt = w.algorithmic_bytes("fwd+bwd") / w.elements
+    return {"value": round(per_elt * elements / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{w.op} eager bf16 fwd+autograd bwd on x{list(t['x'].shape)} (first {sample_rows} rows of the "
                       f"workload), median of {len(times)} runs, {med * 1e3:.1f} ms/run, "
-                      f"{t['x'].numel() // w.cols / med:.3e} rows/s, 10 B/element"}
+                      f"{t['x'].numel() // w.cols / med:.3e} rows/s, {per_elt:.0f} B/element"}
 
 
 def measure(w, steps, warmup):

@@ -58,3 +58,14 @@ def eager_adaln_fwd_bwd(x, scale, shift, dy, eps):
     y = mod(xr, sh, sc)
     y.backward(dy)
     return y.detach(), xr.grad, sc.grad, sh.grad
+
+
+def eager_gate_fwd_bwd(x, gate, residual, dy):
+    """``x + gate * residual`` (GateModule, teletron/models/wan/wan_model.py:205-210) forward +
+    autograd backward; returns (out, dx, dgate, dresidual)."""
+    xr = x.detach().clone().requires_grad_(True)
+    gr = gate.detach().clone().requires_grad_(True)
+    rr = residual.detach().clone().requires_grad_(True)
+    out = xr + gr * rr
+    out.backward(dy)
+    return out.detach(), xr.grad, gr.grad, rr.grad

@@ -6,6 +6,9 @@ ships no code that performs the swap.  This module does it by patching *instance
 * every ``RMSNorm``-style module (``weight`` + ``eps`` + ``norm`` method, as in
   ``teletron/models/wan/wan_model.py:113-124``) gets a fused ``forward``; parameters and
   state-dict keys are untouched;
+* every ``GateModule`` / ``ContextParallelGateModule`` (``x + gate * residual``,
+  ``wan_model.py:205-210``, ``core/context_parallel/layers.py:12-36``) gets the fused gated
+  residual add;
 * every ``nn.LayerNorm(dim, eps, elementwise_affine=False)`` that feeds a modulation
   (``norm1`` / ``norm2`` of ``DiTBlock`` and ``ContextParallelWanDitBlock``, ``norm`` of
   ``Head`` and of the HunyuanVideo ``AdaLayerNormZero[Single]``:
@@ -33,11 +36,12 @@ from typing import Callable, Iterable, Optional
 import torch
 import torch.nn as nn
 
-from .functional import AdaLNModelFunction, RMSNormModelFunction
+from .functional import AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction
 
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
 MODULATE_ATTRS = ("modulate", "modulate_with_cp_grad_reduce")
+GATE_CLASSES = ("GateModule", "ContextParallelGateModule")   # wan_model.py:205-210, context_parallel/layers.py:12-17
 
 
 def fused_kernels_requested() -> bool:
@@ -125,15 +129,22 @@ def _fused_rmsnorm_forward(self, x: torch.Tensor) -> torch.Tensor:
     return type(self).forward(self, x)
 
 
+def _fused_gate_forward(self, x, gate, residual):
+    if x.is_cuda and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 and x.shape == residual.shape:
+        return GateResidualFunction.apply(x, gate, residual)
+    return type(self).forward(self, x, gate, residual)
+
+
 def _is_plain_layernorm(m) -> bool:
     return (isinstance(m, nn.LayerNorm) and not m.elementwise_affine and len(m.normalized_shape) == 1)
 
 
-def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool = True, adaln: bool = True) -> dict:
+def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool = True, adaln: bool = True,
+            gate: bool = True) -> dict:
     """Patch ``model`` in place.  ``namespaces`` are Python modules (e.g. the imported
     ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
     tokens.  Returns counts of what was swapped."""
-    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0}
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0}
     for ns in namespaces:
         fn = getattr(ns, "modulate", None)
         if callable(fn) and not hasattr(fn, "__wrapped__"):
@@ -143,6 +154,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if rmsnorm and _is_rmsnorm(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(_fused_rmsnorm_forward, module)
             counts["rmsnorm"] += 1
+        if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__:
+            module.forward = types.MethodType(_fused_gate_forward, module)
+            counts["gate"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
             for attr in MODULATE_ATTRS:
                 fn = getattr(module, attr, None)

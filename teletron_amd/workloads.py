@@ -15,7 +15,7 @@ import torch
 @dataclass(frozen=True)
 class Workload:
     name: str
-    op: str                      # "adaln" | "rmsnorm"
+    op: str                      # "adaln" | "rmsnorm" | "gate"
     shape: Tuple[int, ...]       # activation shape, normalised dim last
     param_shape: Tuple[int, ...]
     eps: float = 1e-6
@@ -43,6 +43,10 @@ class Workload:
         n_param = 1
         for d in self.param_shape:
             n_param *= d
+        if self.op == "gate":        # out = x + gate * residual: two activations in, one out, each way
+            fwd = 6 * e + n_param * 2
+            bwd = 6 * e + n_param * 2 + n_param * 4
+            return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
         n_vec = 2 if self.op == "adaln" else 1
         fwd = 4 * e + n_vec * n_param * 2
         bwd = 6 * e + n_param * 2 + n_vec * n_param * 4
@@ -56,6 +60,7 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
     Workload("rmsnorm_hunyuan_head", "rmsnorm", (1, 118800, 24, 128), (128,), note="HunyuanVideo per-head norm (per tensor)"),
     Workload("adaln_wan1p3b_batched", "adaln", (4, 32760, 1536), (4, 1, 1536), note="per-sample modulation"),
     Workload("adaln_odd", "adaln", (3, 5000, 1000), (3, 1, 1000), note="125 packs per row: ragged wave tail"),
+    Workload("gate_wan14b", "gate", (1, 75600, 5120), (1, 1, 5120), note="gated residual add after each AdaLN site"),
 ]}
 
 
@@ -71,7 +76,10 @@ def make_inputs(w: Workload, seed: int = 0, device="cpu", rows: Optional[int] = 
     g = torch.Generator(device="cpu").manual_seed(seed)
     x = torch.randn(shape, generator=g, dtype=torch.float32)
     out = {}
-    if w.op == "adaln":
+    if w.op == "gate":
+        out["gate"] = 0.5 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        out["residual"] = torch.randn(shape, generator=g, dtype=torch.float32)
+    elif w.op == "adaln":
         shift = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
         scale = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
         out["shift"], out["scale"] = shift, scale

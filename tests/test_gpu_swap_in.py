@@ -2,6 +2,7 @@
 TeleTron's model code (class names, attribute names, who calls modulate how):
   RMSNorm                  teletron/models/wan/wan_model.py:113-124
   DiTBlock                 wan_model.py:212-243  (module-level modulate(), chunk(6, dim=1) views)
+  GateModule               wan_model.py:205-210
   Head                     wan_model.py:266-278  (inline norm(x) * (1 + scale) + shift)
   AdaLayerNormZeroSingle   teletron/models/hunyuan/model.py:472-504 (self.modulate, [:, None] views)
 The reference itself cannot be imported here (megatron / diffusers are not installed), so the
@@ -41,9 +42,15 @@ class RMSNorm(nn.Module):
         return self.norm(x.float()).to(x.dtype) * self.weight
 
 
+class GateModule(nn.Module):
+    def forward(self, x, gate, residual):
+        return x + gate * residual
+
+
 class DiTBlock(nn.Module):
     def __init__(self, dim, eps=1e-6):
         super().__init__()
+        self.gate, self.gate2 = GateModule(), GateModule()
         self.q, self.k = nn.Linear(dim, dim), nn.Linear(dim, dim)
         self.norm_q, self.norm_k = RMSNorm(dim, eps), RMSNorm(dim, eps)
         self.norm1 = nn.LayerNorm(dim, eps=eps, elementwise_affine=False)
@@ -56,10 +63,10 @@ class DiTBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
             self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
         h = ns.modulate(self.norm1(x), shift_msa, scale_msa)
-        x = x + gate_msa * (self.norm_q(self.q(h)) + self.norm_k(self.k(h)))
+        x = self.gate(x, gate_msa, self.norm_q(self.q(h)) + self.norm_k(self.k(h)))
         x = x + self.norm3(x) * 0.1
         h = ns.modulate(self.norm2(x), shift_mlp, scale_mlp)
-        return x + gate_mlp * self.ffn(h)
+        return self.gate2(x, gate_mlp, self.ffn(h))
 
 
 class Head(nn.Module):
@@ -136,7 +143,7 @@ def test_swap_in_matches_eager_model(monkeypatch):
     assert S.swap_in_if_requested(model, [ns]) is None
     monkeypatch.setenv("FUSED_KERNELS", "1")
     counts = S.swap_in_if_requested(model, [ns])
-    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2}, counts
+    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4}, counts
     assert isinstance(model.blocks[0].norm3, nn.LayerNorm)               # affine LayerNorm untouched
     assert list(model.state_dict().keys()) == keys_before                 # checkpoint compatible
     try:
@@ -150,7 +157,7 @@ def test_swap_in_matches_eager_model(monkeypatch):
         assert rel(a, b) < 2e-2
     worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
     assert worst < 2e-2, worst
-    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1}   # idempotent on the model
+    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0}   # idempotent on the model
 
 
 def test_deferred_norm_refuses_other_uses():
