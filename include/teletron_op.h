@@ -137,6 +137,28 @@ TT_API int tt_rmsnorm_backward_partials(void* dx, const void* dy, const void* x,
 TT_API int tt_reduce_partials(float* out0, float* out1, const void* workspace,
                        int n_batches, int n_partials, int n_acc, int64_t cols, void* stream);
 
+/* ------------------------------------------------------------------ RMSNorm + rotary embedding
+ * The QK-norm of Wan self-attention is followed at once by the rotary position embedding
+ * (norm_q / norm_k then rope_apply: teletron/models/wan/wan_model.py:105-110,154-158), which
+ * the reference runs as separate float64 complex torch ops.  These entry points do both in the
+ * one pass over the tensor:
+ *   t = x * rsqrt(mean(x^2) + eps) * weight                         (full hidden dimension)
+ *   (y[2i], y[2i+1]) = (t[2i] + i t[2i+1]) * (cos + i sin)          per head, pair by pair
+ * freqs is fp32 [seq_len][head_dim / 2][2] = (cos, sin) for position and complex index inside a
+ * head (the reference's complex freqs[s, 1, head_dim / 2] viewed as real); row r uses position
+ * r % seq_len, every head of a row the same table.  Backward multiplies dy by the conjugate and
+ * continues as tt_rmsnorm_backward.  Requires cols % head_dim == 0, head_dim % 8 == 0,
+ * cols > 256, 16-byte aligned tensors (TT_ERR_UNSUPPORTED otherwise).  Workspace as for
+ * tt_rmsnorm_backward.  No counterpart in teletron_op.
+ */
+TT_API int tt_rmsnorm_rope_forward(void* y, const void* x, const void* weight, const float* freqs, float* rstd,
+                                   int64_t rows, int64_t cols, int64_t head_dim, int64_t seq_len,
+                                   float eps, void* stream);
+TT_API int tt_rmsnorm_rope_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
+                                    const float* freqs, void* workspace, size_t workspace_bytes,
+                                    int64_t rows, int64_t cols, int64_t head_dim, int64_t seq_len,
+                                    float eps, void* stream);
+
 /* ------------------------------------------------------------------ gated residual add
  * out = x + gate * residual, the op that follows each fused AdaLN site in a DiT block;
  * gate is [n_batches, cols] bf16, broadcast over the rows of its batch.  teletron_op has no

@@ -174,6 +174,39 @@ def rmsnorm_backward_from_saved(dy, y, gamma, rstd):
     return dx.reshape(y.shape), (dyf * xh).sum(dim=0)
 
 
+# --------------------------------------------------------------------------- rotary embedding behind RMSNorm
+def rope_apply(t, freqs_cs, head_dim: int):
+    """Rotary embedding of teletron/models/wan/wan_model.py:105-110 written on real pairs:
+    inside every head, (t[2i], t[2i+1]) is multiplied as a complex number by
+    (cos, sin) = freqs_cs[position, i].  ``t`` is [..., S, C] with C a multiple of
+    ``head_dim``; ``freqs_cs`` is [S, head_dim/2, 2]; leading dims broadcast over positions."""
+    tf = _f64(t)
+    s, c = tf.shape[-2], tf.shape[-1]
+    f = _f64(freqs_cs).reshape(s, 1, head_dim // 2, 2)
+    v = tf.reshape(*tf.shape[:-1], c // head_dim, head_dim // 2, 2)
+    re = v[..., 0] * f[..., 0] - v[..., 1] * f[..., 1]
+    im = v[..., 0] * f[..., 1] + v[..., 1] * f[..., 0]
+    return torch.stack([re, im], dim=-1).reshape(tf.shape)
+
+
+def rope_apply_backward(dy, freqs_cs, head_dim: int):
+    """Gradient of ``rope_apply`` w.r.t. its input: multiplication by the conjugate."""
+    f = _f64(freqs_cs).clone()
+    f[..., 1] = -f[..., 1]
+    return rope_apply(dy, f, head_dim)
+
+
+def rmsnorm_rope_forward(x, gamma, freqs_cs, eps: float, head_dim: int):
+    """rope_apply(rmsnorm(x) * gamma): norm_q / norm_k followed by rope_apply (wan_model.py:154-158)."""
+    y, _, rstd = rmsnorm_forward(x, gamma, eps)
+    return rope_apply(y, freqs_cs, head_dim), rstd
+
+
+def rmsnorm_rope_backward(dy, x, gamma, freqs_cs, eps: float, head_dim: int):
+    """(dx, dgamma) of the above: un-rotate dy, then the RMSNorm backward."""
+    return rmsnorm_backward(rope_apply_backward(dy, freqs_cs, head_dim), x, gamma, eps)
+
+
 # --------------------------------------------------------------------------- gated residual add
 def gate_residual_forward(x, gate, residual, n_batches: int = 1):
     """out = x + gate * residual (teletron/models/wan/wan_model.py:205-210); gate [B, C]."""

@@ -52,6 +52,10 @@ PROTOTYPES = {
                                              c_void_p, c_size_t, POINTER(c_int),
                                              c_int64, c_int64, c_float, c_void_p]),
     "tt_reduce_partials": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
+    "tt_rmsnorm_rope_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_rmsnorm_rope_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                         c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_gate_residual_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "tt_gate_residual_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                           c_int64, c_int64, c_int64, c_void_p]),

@@ -67,6 +67,11 @@ std::atomic<int> g_grid_override{0};
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+struct Rope {
+  const float* freqs = nullptr;
+  int64_t head_dim = 0, seq_len = 0;
+};
+
 struct Plan {
   KernelInfo k;
   int64_t n_batches = 0;
@@ -81,7 +86,7 @@ constexpr int kGateKind = 2;   // third op family next to kAdaLN / kRMS
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
 constexpr int kMaxWgsPerCu = 8;
 
-int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan) {
+int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan, bool rope = false) {
   if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0)
     return TT_ERR_INVALID_ARGUMENT;
   if (cols > TT_MAX_COLS) return TT_ERR_UNSUPPORTED;
@@ -93,7 +98,10 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   const int slots = narrow ? kNarrowL[idx] : 64 * kWideW[idx] * kWideP[idx];
   const bool full = (slots == packs);
   KernelInfo k;
-  if (kind == kAdaLN)
+  if (rope) {
+    if (narrow || kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
+    k = rms_rope_kernel(dir == kBwd, idx, full);
+  } else if (kind == kAdaLN)
     k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
   else if (kind == kRMS)
@@ -245,16 +253,28 @@ bool vector_path(int64_t cols, std::initializer_list<const void*> ptrs) {
   return true;
 }
 
+int check_rope(const Rope& rope, int64_t cols) {
+  if (!rope.freqs || rope.head_dim <= 0 || rope.seq_len <= 0) return TT_ERR_INVALID_ARGUMENT;
+  if (rope.head_dim % kPack != 0 || cols % rope.head_dim != 0 || !aligned16(rope.freqs)) return TT_ERR_UNSUPPORTED;
+  return TT_OK;
+}
+
 int forward(int kind, void* y, const void* x, const void* p0, const void* p1, float* mean, float* rstd, void* x_norm,
-            int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+            int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream, const Rope* rope = nullptr) {
   if (rows == 0) return TT_OK;
   if (!y || !x || !p0 || (kind == kAdaLN && !p1)) return TT_ERR_INVALID_ARGUMENT;
-  if (!vector_path(cols, {y, x, p0, p1, x_norm}))
+  if (rope) {
+    if (!vector_path(cols, {y, x, p0})) return TT_ERR_UNSUPPORTED;
+    const int rrc = check_rope(*rope, cols);
+    if (rrc != TT_OK) return rrc;
+  } else if (!vector_path(cols, {y, x, p0, p1, x_norm})) {
     return forward_generic(kind, y, x, p0, p1, mean, rstd, x_norm, rows, cols, rows_per_batch, eps, stream);
+  }
   Plan p;
-  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p);
+  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p, rope != nullptr);
   if (rc != TT_OK) return rc;
   FwdArgs a;
+  a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
   a.y = y; a.x = x; a.p0 = p0; a.p1 = p1; a.mean = mean; a.rstd = rstd; a.x_norm = x_norm;
   a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
   a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
@@ -263,17 +283,23 @@ int forward(int kind, void* y, const void* x, const void* p0, const void* p1, fl
 
 int backward_partials(int kind, void* dx, const void* dy, const void* x, const void* p0,
                       void* workspace, size_t workspace_bytes, int* n_partials,
-                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream,
+                      const Rope* rope = nullptr) {
   if (n_partials) *n_partials = 0;
   if (rows == 0) return TT_OK;
   if (!dx || !dy || !x || !p0) return TT_ERR_INVALID_ARGUMENT;
   if (!aligned16(dx) || !aligned16(dy) || !aligned16(x) || !aligned16(p0)) return TT_ERR_UNSUPPORTED;
+  if (rope) {
+    const int rrc = check_rope(*rope, cols);
+    if (rrc != TT_OK) return rrc;
+  }
   Plan p;
-  int rc = make_plan(kind, kBwd, rows, cols, rows_per_batch, &p);
+  int rc = make_plan(kind, kBwd, rows, cols, rows_per_batch, &p, rope != nullptr);
   if (rc != TT_OK) return rc;
   const int n_acc = kind == kAdaLN ? 2 : 1;
   if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;
   BwdArgs a;
+  a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
   a.dx = dx; a.dy = dy; a.x = x; a.p0 = p0; a.partials = static_cast<float*>(workspace);
   a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
   a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
@@ -409,6 +435,26 @@ int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x,
   int n_partials = 0;
   int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
                              rows, cols, rows, eps, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, false, stream);
+}
+
+// ---------------------------------------------------------------- RMSNorm + rotary embedding
+int tt_rmsnorm_rope_forward(void* y, const void* x, const void* weight, const float* freqs, float* rstd,
+                            int64_t rows, int64_t cols, int64_t head_dim, int64_t seq_len, float eps, void* stream) {
+  Rope rope; rope.freqs = freqs; rope.head_dim = head_dim; rope.seq_len = seq_len;
+  return forward(kRMS, y, x, weight, nullptr, nullptr, rstd, nullptr, rows, cols, rows, eps, stream, &rope);
+}
+
+int tt_rmsnorm_rope_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
+                             const float* freqs, void* workspace, size_t workspace_bytes,
+                             int64_t rows, int64_t cols, int64_t head_dim, int64_t seq_len, float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dweight) return TT_ERR_INVALID_ARGUMENT;
+  Rope rope; rope.freqs = freqs; rope.head_dim = head_dim; rope.seq_len = seq_len;
+  int n_partials = 0;
+  int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
+                             rows, cols, rows, eps, stream, &rope);
   if (rc != TT_OK) return rc;
   return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, false, stream);
 }

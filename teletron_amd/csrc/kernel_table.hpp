@@ -157,6 +157,29 @@ KernelInfo lookup_bwd(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
+// RMSNorm with the rotary embedding fused behind it (wide rows only).
+template <int W, int P, bool FULL>
+KernelInfo info_fwd_rope_wide() {
+  constexpr int R = fwd_wide_R(W, P), Q = fwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_fwd_wide<kRMS, W, P, R, Q, FULL, true>), 64 * W * Q, Q * R, P * R};
+}
+template <int W, int P, bool FULL>
+KernelInfo info_bwd_rope_wide() {
+  constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_bwd_wide<kRMS, W, P, R, Q, FULL, true>), 64 * W * Q, Q * R, P * R};
+}
+inline KernelInfo lookup_rope(bool backward, int idx, bool full) {
+  switch (idx) {
+#define X(i, W, P)                                                                                  \
+  case i:                                                                                           \
+    return backward ? (full ? info_bwd_rope_wide<W, P, true>() : info_bwd_rope_wide<W, P, false>()) \
+                    : (full ? info_fwd_rope_wide<W, P, true>() : info_fwd_rope_wide<W, P, false>());
+    TT_WIDE_LIST(X)
+#undef X
+  }
+  return {nullptr, 0, 0, 0};
+}
+
 template <int MODE, int W, int P, bool FULL>
 KernelInfo info_gate_wide() {
   constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
@@ -203,13 +226,14 @@ KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
-// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, gate.hip).
+// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, rms_rope.hip, gate.hip).
 KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_saved_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
+KernelInfo rms_rope_kernel(bool backward, int idx, bool full);
 KernelInfo gate_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo gate_bwd_kernel(bool narrow, int idx, bool full);
 

@@ -44,6 +44,11 @@ struct FwdArgs {
   int packs;        // cols / 8
   float eps;
   float inv_cols;
+  // rotary embedding fused behind RMSNorm (ROPE kernels only): (cos, sin) per position and
+  // complex index of a head, fp32 [seq_len][head_dim / 2][2]; row r sits at position r % seq_len
+  const float* freqs;
+  int64_t seq_len;
+  int head_dim;
 };
 
 struct BwdArgs {
@@ -58,7 +63,35 @@ struct BwdArgs {
   int packs;
   float eps;
   float inv_cols;
+  const float* freqs;   // as in FwdArgs (ROPE kernels only)
+  int64_t seq_len;
+  int head_dim;
 };
+
+// Rotary helpers: a pack holds 4 (re, im) pairs; fr holds their 4 (cos, sin) pairs.
+__device__ __forceinline__ void rope_rotate(float (&v)[8], const float (&fr)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float re = v[2 * k], im = v[2 * k + 1], c = fr[2 * k], sn = fr[2 * k + 1];
+    v[2 * k] = fmaf(re, c, -im * sn);
+    v[2 * k + 1] = fmaf(re, sn, im * c);
+  }
+}
+// Multiplication by the conjugate: the gradient of rope_rotate with respect to its input.
+__device__ __forceinline__ void rope_unrotate(float (&v)[8], const float (&fr)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float re = v[2 * k], im = v[2 * k + 1], c = fr[2 * k], sn = fr[2 * k + 1];
+    v[2 * k] = fmaf(re, c, im * sn);
+    v[2 * k + 1] = fmaf(im, c, -re * sn);
+  }
+}
+__device__ __forceinline__ void load_freq8(const float* freqs, size_t off, float (&fr)[8]) {
+  const f32x4* p = reinterpret_cast<const f32x4*>(freqs + off);
+  const f32x4 a = p[0], b = p[1];
+  fr[0] = a[0]; fr[1] = a[1]; fr[2] = a[2]; fr[3] = a[3];
+  fr[4] = b[0]; fr[5] = b[1]; fr[6] = b[2]; fr[7] = b[3];
+}
 
 // Sum NV values over the W waves of one row group.  `buf` points at W*NV floats
 // of LDS private to (reduction phase parity, row group).  Callers alternate two
@@ -86,9 +119,10 @@ __device__ __forceinline__ void rowgroup_allsum(float (&v)[NV], float* buf, int 
 }
 
 // ============================================================================ wide forward
-template <int KIND, int W, int P, int R, int Q, bool FULL>
+template <int KIND, int W, int P, int R, int Q, bool FULL, bool ROPE = false>
 __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
+  static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
   __shared__ float red[2][Q][W * R];
 
   const int lane = threadIdx.x & 63;
@@ -124,6 +158,12 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   // issued before the arithmetic of the current one, so every wave keeps a tile
   // in flight while it computes.
   u32x4 raw[R][P];
+  float fr[ROPE ? R : 1][ROPE ? P : 1][8];   // (cos, sin) of the packs being fetched
+  int fcol[P];                               // column inside its head
+  if constexpr (ROPE) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) fcol[p] = col[p] % a.head_dim;
+  }
   auto fetch = [&](int64_t t) {
     const int64_t r0 = t * (Q * R) + q * R;
 #pragma unroll
@@ -131,7 +171,15 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
 #pragma unroll
       for (int p = 0; p < P; ++p) {
         raw[r][p] = u32x4{0, 0, 0, 0};
-        if (r0 + r < S && act[p]) raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
+        if constexpr (ROPE) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) fr[r][p][j] = 0.f;
+        }
+        if (r0 + r < S && act[p]) {
+          raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
+          if constexpr (ROPE)
+            load_freq8(a.freqs, (size_t)(((b * S + r0 + r) % a.seq_len) * a.head_dim + fcol[p]), fr[r][p]);
+        }
       }
   };
 
@@ -148,6 +196,15 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
       rv[r] = row0 + r < S;
 #pragma unroll
       for (int p = 0; p < P; ++p) unpack8(raw[r][p], xf[r][p]);
+    }
+    float fc[ROPE ? R : 1][ROPE ? P : 1][8];
+    if constexpr (ROPE) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) fc[r][p][j] = fr[r][p][j];
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 
@@ -207,6 +264,7 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
               n[j] = xh;
               o[j] = ADALN ? fmaf(xh, g[p][j], sh[p][j]) : xh * g[p][j];
             }
+            if constexpr (ROPE) rope_rotate(o, fc[r][p]);
             store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
             if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col[p]), pack8(n));
           }
@@ -272,9 +330,10 @@ __device__ __forceinline__ void wide_write_partials(float (&acc0)[P][8], float (
 }
 
 // ============================================================================ wide backward
-template <int KIND, int W, int P, int R, int Q, bool FULL>
+template <int KIND, int W, int P, int R, int Q, bool FULL, bool ROPE = false>
 __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
+  static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
   constexpr int NACC = ADALN ? 2 : 1;
   constexpr int NV = ADALN ? 3 : 2;  // reduced values per row in the main phase
   __shared__ float red[2][Q][W * R * NV];
@@ -309,6 +368,12 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
   }
 
   u32x4 rawx[R][P], rawd[R][P];
+  float fr[ROPE ? R : 1][ROPE ? P : 1][8];
+  int fcol[P];
+  if constexpr (ROPE) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) fcol[p] = col[p] % a.head_dim;
+  }
   auto fetch = [&](int64_t t) {
     const int64_t r0 = t * (Q * R) + q * R;
 #pragma unroll
@@ -317,10 +382,16 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
       for (int p = 0; p < P; ++p) {
         rawx[r][p] = u32x4{0, 0, 0, 0};
         rawd[r][p] = u32x4{0, 0, 0, 0};
+        if constexpr (ROPE) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) fr[r][p][j] = 0.f;
+        }
         if (r0 + r < S && act[p]) {
           const size_t off = (size_t)((b * S + r0 + r) * C + col[p]);
           rawx[r][p] = load_stream(a.x, off);
           rawd[r][p] = load_stream(a.dy, off);
+          if constexpr (ROPE)
+            load_freq8(a.freqs, (size_t)(((b * S + r0 + r) % a.seq_len) * a.head_dim + fcol[p]), fr[r][p]);
         }
       }
   };
@@ -340,6 +411,8 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
       for (int p = 0; p < P; ++p) {
         unpack8(rawx[r][p], xf[r][p]);
         unpack8(rawd[r][p], df[r][p]);
+        // the incoming gradient is that of the rotated output: undo the rotation first
+        if constexpr (ROPE) rope_unrotate(df[r][p], fr[r][p]);
       }
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);

@@ -75,6 +75,33 @@ class RMSNormModelFunction(Function):
         return dx, dweight, None, None
 
 
+class RMSNormRopeFunction(Function):
+    """``rope_apply(RMSNorm(x), freqs, num_heads)`` (``teletron/models/wan/wan_model.py:105-110,154-158``)
+    as one op.  ``freqs`` is the model's complex ``[S, 1, head_dim/2]`` table (or real
+    ``[S, head_dim/2, 2]`` cos/sin); it gets no gradient."""
+
+    @staticmethod
+    def forward(ctx, x, weight, freqs, epsilon, num_heads):
+        cols = x.shape[-1]
+        if cols % num_heads != 0:
+            raise ValueError(f"hidden size {cols} not divisible by num_heads {num_heads}")
+        ctx.eps, ctx.head_dim = float(epsilon), cols // num_heads
+        ctx.weight_meta = (weight.shape, weight.dtype)
+        x = x.contiguous()
+        weight_c = weight.detach().to(torch.bfloat16).contiguous()
+        freqs_c = ops._check_freqs(freqs.detach(), x, ctx.head_dim)
+        ctx.save_for_backward(x, weight_c, freqs_c)
+        return ops.rmsnorm_rope_forward(x, weight_c, freqs_c, ctx.eps, ctx.head_dim)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight_c, freqs_c = ctx.saved_tensors
+        dx, dweight = ops.rmsnorm_rope_backward(grad_output.contiguous(), x, weight_c, freqs_c, ctx.eps, ctx.head_dim)
+        w_shape, w_dtype = ctx.weight_meta
+        return (dx if ctx.needs_input_grad[0] else None,
+                dweight.to(w_dtype).reshape(w_shape) if ctx.needs_input_grad[1] else None, None, None, None)
+
+
 class GateResidualFunction(Function):
     """``x + gate * residual`` with the hand-written backward of ``GateWithGradReduce``
     (``teletron/core/context_parallel/layers.py:24-36``) on one GPU: returns

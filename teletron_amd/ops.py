@@ -184,3 +184,54 @@ def gate_residual_backward(dout: torch.Tensor, gate: torch.Tensor, residual: tor
         cabi.call("tt_gate_residual_backward", dres.data_ptr(), dgate.data_ptr(), dout.data_ptr(), gate.data_ptr(),
                   residual.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, rpb, _stream(dout))
     return dres, dgate
+
+
+def _check_freqs(freqs: torch.Tensor, x: torch.Tensor, head_dim: int) -> torch.Tensor:
+    """freqs: real [S, head_dim/2, 2] (cos, sin), or the reference's complex [S, 1, head_dim/2]."""
+    _require(isinstance(freqs, torch.Tensor) and freqs.device == x.device, ValueError, "freqs must be on the input's device")
+    if freqs.is_complex():
+        freqs = torch.view_as_real(freqs.to(torch.complex64))
+    freqs = freqs.to(torch.float32).reshape(-1, head_dim // 2, 2).contiguous()
+    return freqs
+
+
+def rmsnorm_rope_forward(x: torch.Tensor, weight: torch.Tensor, freqs: torch.Tensor, eps: float, head_dim: int):
+    """rope(rmsnorm(x) * weight) in one pass.  x: [..., S, C] bf16 with S = freqs.shape[0] positions."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    weight = _check_param("weight", weight, x, cols)
+    _require(weight.numel() == cols, ValueError, f"weight must have {cols} elements, got {weight.numel()}")
+    _require(head_dim > 0 and cols % head_dim == 0 and head_dim % 2 == 0, ValueError,
+             f"head_dim {head_dim} must be even and divide cols {cols}")
+    freqs = _check_freqs(freqs, x, head_dim)
+    rows, seq = x.numel() // cols, freqs.shape[0]
+    _require(x.dim() >= 2 and x.shape[-2] == seq, ValueError,
+             f"x has {x.shape[-2] if x.dim() >= 2 else 1} positions, freqs {seq}")
+    y = torch.empty_like(x)
+    if rows:
+        with torch.cuda.device(x.device):
+            cabi.call("tt_rmsnorm_rope_forward", y.data_ptr(), x.data_ptr(), weight.data_ptr(), freqs.data_ptr(), None,
+                      rows, cols, head_dim, seq, float(eps), _stream(x))
+    return y
+
+
+def rmsnorm_rope_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, freqs: torch.Tensor,
+                          eps: float, head_dim: int):
+    """Returns (dx bf16 like x, dweight fp32 [C]) for y = rope(rmsnorm(x) * weight)."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    dy = _check_act("dy", dy, cols)
+    _require(dy.numel() == x.numel() and dy.device == x.device, ValueError, "dy must match x in size and device")
+    weight = _check_param("weight", weight, x, cols)
+    freqs = _check_freqs(freqs, x, head_dim)
+    rows, seq = x.numel() // cols, freqs.shape[0]
+    dx = torch.empty_like(x)
+    if rows == 0:
+        return dx, torch.zeros(cols, dtype=torch.float32, device=x.device)
+    dweight = torch.empty(cols, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        ws = _workspace(cabi.load().tt_rmsnorm_backward_workspace_bytes(rows, cols), 0, x)
+        cabi.call("tt_rmsnorm_rope_backward", dx.data_ptr(), dweight.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                  weight.data_ptr(), freqs.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, head_dim, seq,
+                  float(eps), _stream(x))
+    return dx, dweight

@@ -220,6 +220,33 @@ def test_saved_tensor_backward_equals_backward_from_x():
     torch.testing.assert_close(dgamma2, dgamma, rtol=1e-11, atol=1e-12)
 
 
+def test_rope_matches_complex_arithmetic_and_autograd():
+    # independent route: torch's complex multiply, laid out as in wan_model.py:105-110
+    b, s, n, d, eps = 2, 7, 3, 16, 1e-6
+    c = n * d
+    x = rnd(b, s, c, seed=60).requires_grad_(True)
+    gamma = (1 + rnd(c, seed=61, scale=0.2)).requires_grad_(True)
+    ang = rnd(s, d // 2, seed=62, scale=2.0)
+    freqs = torch.polar(torch.ones_like(ang), ang).reshape(s, 1, d // 2)           # complex128 [s, 1, d/2]
+    freqs_cs = torch.view_as_real(freqs).reshape(s, d // 2, 2)
+    dy = rnd(b, s, c, seed=63)
+    t = F.rms_norm(x, (c,), weight=gamma, eps=eps)
+    out = torch.view_as_real(torch.view_as_complex(t.reshape(b, s, n, d // 2, 2)) * freqs).flatten(2)
+    y, _ = O.rmsnorm_rope_forward(x, gamma, freqs_cs, eps, d)
+    torch.testing.assert_close(y, out.detach(), rtol=1e-12, atol=1e-12)
+    out.backward(dy)
+    dx, dgamma = O.rmsnorm_rope_backward(dy, x, gamma, freqs_cs, eps, d)
+    torch.testing.assert_close(dx, x.grad, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(dgamma, gamma.grad, rtol=1e-10, atol=1e-12)
+    # a rotation keeps the modulus of every pair, and angle 0 is the identity
+    t0 = rnd(b, s, c, seed=64)
+    r = O.rope_apply(t0, freqs_cs, d).reshape(b, s, c // 2, 2)
+    torch.testing.assert_close(r.pow(2).sum(-1), t0.reshape(b, s, c // 2, 2).pow(2).sum(-1), rtol=1e-12, atol=1e-12)
+    ident = torch.stack([torch.ones(s, d // 2), torch.zeros(s, d // 2)], dim=-1)
+    torch.testing.assert_close(O.rope_apply(t0, ident, d), t0, rtol=0, atol=0)
+    torch.testing.assert_close(O.rope_apply_backward(O.rope_apply(t0, freqs_cs, d), freqs_cs, d), t0, rtol=1e-12, atol=1e-12)
+
+
 def test_gate_residual_matches_autograd():
     nb, s, c = 3, 5, 24
     x, r, dy = rnd(nb, s, c, seed=50).requires_grad_(True), rnd(nb, s, c, seed=51).requires_grad_(True), rnd(nb, s, c, seed=52)
