@@ -77,7 +77,13 @@ class GpuWorkload:
                  "y": torch.empty(self.rows, self.cols, dtype=bf, device=dev),
                  "dx": torch.empty(self.rows, self.cols, dtype=bf, device=dev)}
             self.sets.append(s)
-        if w.op == "gate":
+        if w.op == "rope":
+            self.p0 = randn(self.cols, scale=0.1, offset=1.0)              # gamma
+            ang = 3.0 * torch.randn(w.shape[-2], w.head_dim // 2, generator=g, device=dev, dtype=torch.float32)
+            self.p1 = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()   # fp32 (cos, sin) table
+            self.n_acc = 1
+            ws_bytes = self.lib.tt_rmsnorm_backward_workspace_bytes(self.rows, self.cols)
+        elif w.op == "gate":
             # x / dy double as (x, residual) forward and (dout, residual) backward
             self.p0 = randn(self.nb, self.cols, scale=0.5)                 # gate
             self.p1 = None
@@ -101,7 +107,11 @@ class GpuWorkload:
 
     def fwd(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "gate":
+        if self.w.op == "rope":
+            self.cabi.call("tt_rmsnorm_rope_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
+                           self.p1.data_ptr(), None, self.rows, self.cols, self.w.head_dim, self.w.shape[-2],
+                           self.w.eps, self.stream)
+        elif self.w.op == "gate":
             self.cabi.call("tt_gate_residual_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
                            s["dy"].data_ptr(), self.rows, self.cols, self.rpb, self.stream)
         elif self.w.op == "adaln":
@@ -113,7 +123,12 @@ class GpuWorkload:
 
     def bwd_partials(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "gate":          # one entry point: streaming kernel + reduction of its partials
+        if self.w.op == "rope":          # one entry point: streaming kernel + reduction of its partials
+            self.cabi.call("tt_rmsnorm_rope_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
+                           s["x"].data_ptr(), self.p0.data_ptr(), self.p1.data_ptr(), self.ws.data_ptr(),
+                           self.ws.numel(), self.rows, self.cols, self.w.head_dim, self.w.shape[-2], self.w.eps,
+                           self.stream)
+        elif self.w.op == "gate":          # one entry point: streaming kernel + reduction of its partials
             self.cabi.call("tt_gate_residual_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
                            self.p0.data_ptr(), s["x"].data_ptr(), self.ws.data_ptr(), self.ws.numel(),
                            self.rows, self.cols, self.rpb, self.stream)
@@ -127,7 +142,7 @@ class GpuWorkload:
                            self.rows, self.cols, self.w.eps, self.stream)
 
     def reduce(self):
-        if self.w.op == "gate":
+        if self.w.op in ("gate", "rope"):
             return
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
@@ -177,7 +192,9 @@ def cpu_baseline(w, seconds):
     sample_rows = min(w.shape[1], 16384)
     t = make_inputs(w, seed=0, rows=sample_rows)
     elements = t["x"].numel()
-    if w.op == "gate":
+    if w.op == "rope":
+        fn = lambda: E.eager_rmsnorm_rope_fwd_bwd(t["x"], t["gamma"], t["freqs"], t["dy"], w.eps, w.head_dim)
+    elif w.op == "gate":
         fn = lambda: E.eager_gate_fwd_bwd(t["x"], t["gate"], t["residual"], t["dy"])
     elif w.op == "adaln":
         fn = lambda: E.eager_adaln_fwd_bwd(t["x"], t["scale"], t["shift"], t["dy"], w.eps)

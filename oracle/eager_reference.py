@@ -69,3 +69,23 @@ def eager_gate_fwd_bwd(x, gate, residual, dy):
     out = xr + gr * rr
     out.backward(dy)
     return out.detach(), xr.grad, gr.grad, rr.grad
+
+
+def eager_rope_apply(x, freqs, num_heads):
+    """rope_apply of teletron/models/wan/wan_model.py:105-110: float64 complex multiply per head.
+    ``freqs`` is complex [S, 1, head_dim/2]."""
+    b, s, c = x.shape
+    xc = torch.view_as_complex(x.to(torch.float64).reshape(b, s, num_heads, -1, 2))
+    return torch.view_as_real(xc * freqs).flatten(2).to(x.dtype)
+
+
+def eager_rmsnorm_rope_fwd_bwd(x, gamma, freqs_cs, dy, eps, head_dim):
+    """norm_q(x) then rope_apply, as in SelfAttention.forward (wan_model.py:153-158), forward +
+    autograd backward; ``freqs_cs`` is real [S, head_dim/2, 2].  Returns (y, dx, dgamma)."""
+    freqs = torch.view_as_complex(freqs_cs.to(torch.float64).contiguous()).unsqueeze(1)
+    mod = EagerRMSNorm(x.shape[-1], eps)
+    mod.weight = nn.Parameter(gamma.detach().clone())
+    xr = x.detach().clone().requires_grad_(True)
+    y = eager_rope_apply(mod(xr), freqs, x.shape[-1] // head_dim)
+    y.backward(dy)
+    return y.detach(), xr.grad, mod.weight.grad

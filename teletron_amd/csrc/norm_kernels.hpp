@@ -160,12 +160,27 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   u32x4 raw[R][P];
   float fr[ROPE ? R : 1][ROPE ? P : 1][8];   // (cos, sin) of the packs being fetched
   int fcol[P];                               // column inside its head
+  // Position of the first row of the tile that fetch() takes next, kept incrementally:
+  // tiles are fetched in the order blockIdx.x, blockIdx.x + gridDim.x, ...
+  int64_t fpos = 0, fstep = 0;
   if constexpr (ROPE) {
 #pragma unroll
     for (int p = 0; p < P; ++p) fcol[p] = col[p] % a.head_dim;
+    fpos = (b * S + (int64_t)blockIdx.x * (Q * R) + q * R) % a.seq_len;
+    fstep = ((int64_t)gridDim.x * (Q * R)) % a.seq_len;
   }
   auto fetch = [&](int64_t t) {
     const int64_t r0 = t * (Q * R) + q * R;
+    int64_t pos[R];
+    if constexpr (ROPE) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        pos[r] = fpos + r;
+        while (pos[r] >= a.seq_len) pos[r] -= a.seq_len;
+      }
+      fpos += fstep;
+      if (fpos >= a.seq_len) fpos -= a.seq_len;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -178,7 +193,7 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
         if (r0 + r < S && act[p]) {
           raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
           if constexpr (ROPE)
-            load_freq8(a.freqs, (size_t)(((b * S + r0 + r) % a.seq_len) * a.head_dim + fcol[p]), fr[r][p]);
+            load_freq8(a.freqs, (size_t)(pos[r] * a.head_dim + fcol[p]), fr[r][p]);
         }
       }
   };
@@ -370,12 +385,25 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
   u32x4 rawx[R][P], rawd[R][P];
   float fr[ROPE ? R : 1][ROPE ? P : 1][8];
   int fcol[P];
+  int64_t fpos = 0, fstep = 0;   // as in the forward kernel
   if constexpr (ROPE) {
 #pragma unroll
     for (int p = 0; p < P; ++p) fcol[p] = col[p] % a.head_dim;
+    fpos = (b * S + (int64_t)blockIdx.x * (Q * R) + q * R) % a.seq_len;
+    fstep = ((int64_t)gridDim.x * (Q * R)) % a.seq_len;
   }
   auto fetch = [&](int64_t t) {
     const int64_t r0 = t * (Q * R) + q * R;
+    int64_t pos[R];
+    if constexpr (ROPE) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        pos[r] = fpos + r;
+        while (pos[r] >= a.seq_len) pos[r] -= a.seq_len;
+      }
+      fpos += fstep;
+      if (fpos >= a.seq_len) fpos -= a.seq_len;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -391,7 +419,7 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
           rawx[r][p] = load_stream(a.x, off);
           rawd[r][p] = load_stream(a.dy, off);
           if constexpr (ROPE)
-            load_freq8(a.freqs, (size_t)(((b * S + r0 + r) % a.seq_len) * a.head_dim + fcol[p]), fr[r][p]);
+            load_freq8(a.freqs, (size_t)(pos[r] * a.head_dim + fcol[p]), fr[r][p]);
         }
       }
   };

@@ -15,11 +15,12 @@ import torch
 @dataclass(frozen=True)
 class Workload:
     name: str
-    op: str                      # "adaln" | "rmsnorm" | "gate"
+    op: str                      # "adaln" | "rmsnorm" | "rope" | "gate"
     shape: Tuple[int, ...]       # activation shape, normalised dim last
     param_shape: Tuple[int, ...]
     eps: float = 1e-6
     note: str = ""
+    head_dim: int = 0            # "rope" only
 
     @property
     def cols(self) -> int:
@@ -43,6 +44,11 @@ class Workload:
         n_param = 1
         for d in self.param_shape:
             n_param *= d
+        if self.op == "rope":        # RMSNorm + rotary embedding: as rmsnorm plus the fp32 (cos, sin) table, read once
+            table = self.shape[-2] * self.head_dim * 4
+            fwd = 4 * e + n_param * 2 + table
+            bwd = 6 * e + n_param * 2 + n_param * 4 + table
+            return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
         if self.op == "gate":        # out = x + gate * residual: two activations in, one out, each way
             fwd = 6 * e + n_param * 2
             bwd = 6 * e + n_param * 2 + n_param * 4
@@ -60,6 +66,8 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
     Workload("rmsnorm_hunyuan_head", "rmsnorm", (1, 118800, 24, 128), (128,), note="HunyuanVideo per-head norm (per tensor)"),
     Workload("adaln_wan1p3b_batched", "adaln", (4, 32760, 1536), (4, 1, 1536), note="per-sample modulation"),
     Workload("adaln_odd", "adaln", (3, 5000, 1000), (3, 1, 1000), note="125 packs per row: ragged wave tail"),
+    Workload("rmsnorm_rope_wan14b", "rope", (1, 75600, 5120), (5120,), head_dim=128,
+             note="Wan2.1-14B QK-norm + rotary embedding, 40 heads of 128"),
     Workload("gate_wan14b", "gate", (1, 75600, 5120), (1, 1, 5120), note="gated residual add after each AdaLN site"),
 ]}
 
@@ -85,6 +93,12 @@ def make_inputs(w: Workload, seed: int = 0, device="cpu", rows: Optional[int] = 
         out["shift"], out["scale"] = shift, scale
     else:
         out["gamma"] = 1.0 + 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        if w.op == "rope":
+            ang = 3.0 * torch.randn(shape[-2], w.head_dim // 2, generator=g, dtype=torch.float32)
+            freqs = torch.stack([ang.cos(), ang.sin()], dim=-1)
     dy = torch.randn(shape, generator=g, dtype=torch.float32)
     out["x"], out["dy"] = x, dy
-    return {k: v.to(torch.bfloat16).to(device) for k, v in out.items()}
+    out = {k: v.to(torch.bfloat16).to(device) for k, v in out.items()}
+    if w.op == "rope":
+        out["freqs"] = freqs.to(device)          # fp32 [S, head_dim/2, 2]
+    return out
