@@ -46,7 +46,8 @@ def parse_args():
     ap.add_argument("--workload", default="adaln_wan14b")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
-    ap.add_argument("--also", default="rmsnorm_wan14b_qk", help="comma list of further workloads reported under 'also'")
+    ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched",
+                    help="comma list of further workloads reported under 'also'")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
                          "that hardware byte counters collected over this run can be scaled against it")
@@ -229,9 +230,7 @@ def measure(w, steps, warmup):
         "bwd_gbps": w.algorithmic_bytes("bwd") / mean(k["bwd"]) / 1e3,
         "n_partials": g.n_partials.value,
     }
-    del g
-    import torch
-    torch.cuda.empty_cache()
+    del g   # the caching allocator keeps the blocks: later workloads reuse them instead of fresh driver memory
     return res
 
 
