@@ -27,6 +27,22 @@ def sample_rows(n_rows, k, seed):
     return torch.unique(idx)
 
 
+def whole_tensor_check(got, ref_fn, rows_per_block=8192):
+    """Every element of a full-size output against a plain torch fp32 evaluation on the GPU, block
+    of rows by block of rows.  The sampled-row oracle checks above pin the values; this pass is
+    there to catch sparse corruption (a lost or torn store) anywhere in the tensor."""
+    c = got.shape[-1]
+    g2 = got.reshape(-1, c)
+    worst = 0.0
+    for r0 in range(0, g2.shape[0], rows_per_block):
+        ref = ref_fn(r0, min(r0 + rows_per_block, g2.shape[0]))
+        blk = g2[r0:r0 + rows_per_block].float()
+        assert torch.isfinite(blk).all(), f"non-finite output in rows {r0}..{r0 + rows_per_block}"
+        excess = ((blk - ref).abs() - (1e-2 + 8e-3 * ref.abs())).max().item()
+        worst = max(worst, excess)
+    assert worst <= 0, f"whole-tensor check: worst excess over tolerance {worst:.3e}"
+
+
 def test_rmsnorm_small_config_full_oracle():
     from teletron_amd import ops
     w = WORKLOADS["rmsnorm_small"]
@@ -84,6 +100,28 @@ def _adaln_full_size(name, chunk_rows):
     assert_grad_close(dscale, dsco, s, "dscale")
     assert_grad_close(dshift, dsho, s, "dshift")
 
+    # every element, against torch fp32 on the GPU
+    x2, dy2 = xd.reshape(-1, c), dyd.reshape(-1, c)
+
+    def ref_y(r0, r1):
+        b = r0 // s
+        assert (r1 - 1) // s == b or r1 - r0 <= s, "block must not straddle batches unevenly"
+        xs = x2[r0:r1].float()
+        bi = torch.arange(r0, r1, device=DEV) // s
+        xh = torch.nn.functional.layer_norm(xs, (c,), eps=w.eps)
+        return xh * (1 + scd.reshape(nb, c).float()[bi]) + shd.reshape(nb, c).float()[bi]
+
+    def ref_dx(r0, r1):
+        xs, ds = x2[r0:r1].float(), dy2[r0:r1].float()
+        bi = torch.arange(r0, r1, device=DEV) // s
+        xh = torch.nn.functional.layer_norm(xs, (c,), eps=w.eps)
+        rstd = torch.rsqrt(xs.var(-1, unbiased=False, keepdim=True) + w.eps)
+        g = ds * (1 + scd.reshape(nb, c).float()[bi])
+        return rstd * (g - g.mean(-1, keepdim=True) - xh * (g * xh).mean(-1, keepdim=True))
+
+    whole_tensor_check(y, ref_y)
+    whole_tensor_check(dx, ref_dx)
+
     # properties of the whole output
     row_sums = torch.stack([dx[b].float().sum(-1).abs().max() for b in range(nb)]).max().item()
     assert row_sums < 0.02 * math.sqrt(c), f"dx rows should sum to ~0 (bf16 rounding noise only), got {row_sums}"
@@ -122,6 +160,23 @@ def _rmsnorm_full_size(name, chunk_rows):
 
     dgo = O.rmsnorm_backward_param_grads_chunked(dy2, x2, w.eps, chunk_rows)
     assert_grad_close(dgamma, dgo, w.rows, "dgamma")
+
+    # every element, against torch fp32 on the GPU
+    xg2, dyg2, gf = xd.reshape(-1, c), dyd.reshape(-1, c), gd.float()
+
+    def ref_y(r0, r1):
+        xs = xg2[r0:r1].float()
+        return xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + w.eps) * gf
+
+    def ref_dx(r0, r1):
+        xs, ds = xg2[r0:r1].float(), dyg2[r0:r1].float()
+        rstd = torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + w.eps)
+        xh, g = xs * rstd, ds * gf
+        return rstd * (g - xh * (g * xh).mean(-1, keepdim=True))
+
+    blk = 8192 if c > 256 else 1 << 18
+    whole_tensor_check(y, ref_y, blk)
+    whole_tensor_check(dx, ref_dx, blk)
 
     # with gamma == 1 the output rows have mean square ms / (ms + eps) ~ 1: whole-tensor property
     ones = torch.ones_like(gd)

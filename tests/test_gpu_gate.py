@@ -59,6 +59,14 @@ def test_gate_full_size_properties_and_reproducibility():
     for r0 in range(0, rows, 8192):
         ref += (dy[r0:r0 + 8192].cpu().double() * r[r0:r0 + 8192].cpu().double()).sum(0)
     assert_grad_close(dgate, ref, rows, "dgate")
+    # every element against torch fp32 on the GPU (catches sparse corruption anywhere in the tensor)
+    gf = gate.float()
+    for r0 in range(0, rows, 8192):
+        sl = slice(r0, r0 + 8192)
+        ref_o = x[sl].float() + gf * r[sl].float()
+        ref_d = dy[sl].float() * gf
+        assert ((out[sl].float() - ref_o).abs() <= 1e-2 + 8e-3 * ref_o.abs()).all()
+        assert ((dres[sl].float() - ref_d).abs() <= 1e-2 + 8e-3 * ref_d.abs()).all()
     dres2, dgate2 = ops.gate_residual_backward(dy, gate, r)
     assert torch.equal(dres, dres2) and torch.equal(dgate, dgate2)
     # linearity in the gate: out(2g) - out(g) == out(g) - out(0) up to bf16 rounding of the outputs

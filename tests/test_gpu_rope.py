@@ -76,8 +76,13 @@ def test_rope_full_size_rows_and_reproducibility():
     assert_bf16_close(dx[0, di], dxo, "dx rows")
     # a rotation keeps the modulus of each pair: sum y^2 per row == sum (rmsnorm(x) w)^2 per row
     t = ops.rmsnorm_forward(x, w, 1e-6)
-    e1 = y[0, :8192].float().pow(2).sum(-1)
-    e2 = t[0, :8192].float().pow(2).sum(-1)
-    torch.testing.assert_close(e1, e2, rtol=2e-3, atol=0)
+    for r0 in range(0, s, 8192):                      # all rows: also catches sparse corruption
+        e1 = y[0, r0:r0 + 8192].float().pow(2).sum(-1)
+        e2 = t[0, r0:r0 + 8192].float().pow(2).sum(-1)
+        torch.testing.assert_close(e1, e2, rtol=2e-3, atol=0)
+        assert torch.isfinite(dx[0, r0:r0 + 8192].float()).all()
+    # un-rotating dy and running the plain backward must give the same dx as the fused kernel
+    dyu = O.rope_apply_backward(dy[0, di].cpu(), fcs[di].cpu(), hd)
+    assert_bf16_close(dx[0, di], O.rmsnorm_backward(dyu, x[0, di].cpu(), w.cpu(), 1e-6)[0], "dx via unrotate")
     dx2, dw2 = ops.rmsnorm_rope_backward(dy, x, w, fcs, 1e-6, hd)
     assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
