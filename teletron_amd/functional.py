@@ -59,7 +59,8 @@ class RMSNormModelFunction(Function):
             raise ValueError(f"Input size {x.numel()} not divisible by cols {cols}")
         ctx.eps = float(epsilon)
         ctx.weight_meta = (weight.shape, weight.dtype)
-        x = x.contiguous()
+        if ops.memory_order_view(x)[0] is None:      # dense permuted views are handled without a copy
+            x = x.contiguous()
         weight_c = weight.detach().to(torch.bfloat16).contiguous()
         y = ops.rmsnorm_forward(x, weight_c, ctx.eps)
         ctx.save_for_backward(x, weight_c)
@@ -68,7 +69,9 @@ class RMSNormModelFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         x, weight_c = ctx.saved_tensors
-        dx, dweight = ops.rmsnorm_backward(grad_output.contiguous(), x, weight_c, ctx.eps)
+        if x.is_contiguous():
+            grad_output = grad_output.contiguous()
+        dx, dweight = ops.rmsnorm_backward(grad_output, x, weight_c, ctx.eps)
         w_shape, w_dtype = ctx.weight_meta
         dx = dx if ctx.needs_input_grad[0] else None
         dweight = dweight.to(w_dtype).reshape(w_shape) if ctx.needs_input_grad[1] else None

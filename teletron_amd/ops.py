@@ -45,6 +45,27 @@ def _check_param(name: str, p: torch.Tensor, ref: torch.Tensor, cols: int) -> to
     return p.contiguous()
 
 
+def memory_order_view(t: torch.Tensor):
+    """For a dense permuted tensor whose last dimension is contiguous (e.g. the ``[B, H, S, D]``
+    transposed view of a ``[B, S, H, D]`` buffer that HunyuanVideo hands to its per-head norm,
+    ``teletron/models/hunyuan/model.py:87-95``), returns ``(view, perm)`` where ``view`` is ``t``
+    permuted into memory order (contiguous, no copy).  Row-wise ops whose parameters do not depend
+    on the row can run on ``view`` and permute the result back.  Returns ``(None, None)`` when the
+    tensor is already contiguous or is not such a view."""
+    if t.is_contiguous() or t.dim() < 2 or t.stride(-1) != 1:
+        return None, None
+    perm = sorted(range(t.dim() - 1), key=lambda d: -t.stride(d)) + [t.dim() - 1]
+    view = t.permute(perm)
+    return (view, perm) if view.is_contiguous() else (None, None)
+
+
+def _inverse(perm):
+    inv = [0] * len(perm)
+    for i, p in enumerate(perm):
+        inv[p] = i
+    return inv
+
+
 def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int, int]:
     rows = x.numel() // cols
     nb = scale.numel() // cols
@@ -114,7 +135,15 @@ def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: 
 
 
 def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, return_stats: bool = False):
-    """y = x * rsqrt(mean(x^2) + eps) * weight.  Returns y, or (y, rstd)."""
+    """y = x * rsqrt(mean(x^2) + eps) * weight.  Returns y, or (y, rstd).
+
+    A dense permuted input (see ``memory_order_view``) is processed in memory order without a copy
+    and the result has the input's strides; ``rstd`` then follows memory order too."""
+    view, perm = memory_order_view(x) if isinstance(x, torch.Tensor) else (None, None)
+    if view is not None:
+        out = rmsnorm_forward(view, weight, eps, return_stats)
+        inv = _inverse(perm)
+        return (out[0].permute(inv), out[1]) if return_stats else out.permute(inv)
     cols = x.shape[-1]
     x = _check_act("x", x, cols)
     weight = _check_param("weight", weight, x, cols)
@@ -130,7 +159,11 @@ def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, return_st
 
 
 def rmsnorm_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float):
-    """Returns (dx bf16 like x, dweight fp32 [C])."""
+    """Returns (dx bf16 like x, dweight fp32 [C]).  Dense permuted ``x`` as in ``rmsnorm_forward``."""
+    view, perm = memory_order_view(x) if isinstance(x, torch.Tensor) else (None, None)
+    if view is not None and isinstance(dy, torch.Tensor) and dy.shape == x.shape:
+        dx, dweight = rmsnorm_backward(dy.permute(perm), view, weight, eps)
+        return dx.permute(_inverse(perm)), dweight
     cols = x.shape[-1]
     x = _check_act("x", x, cols)
     dy = _check_act("dy", dy, cols)

@@ -287,6 +287,35 @@ def test_autograd_functions_match_oracle():
     assert torch.equal(y3, y.detach())
 
 
+def test_rmsnorm_on_transposed_head_layout_without_a_copy():
+    # HunyuanVideo norms query[B, H, S, D], a transposed view of the [B, S, H, D] projection output
+    from teletron_amd import RMSNormModelFunction, ops
+    b, s, h, d = 2, 203, 24, 128
+    base = rand_bf16(b, s, h, d, seed=60)
+    w = rand_bf16(d, seed=61, scale=0.1, offset=1.0)
+    dy_base = rand_bf16(b, s, h, d, seed=62)
+    xq = base.to(DEV).transpose(1, 2)                      # [B, H, S, D], not contiguous
+    assert not xq.is_contiguous() and ops.memory_order_view(xq)[0] is not None
+    xg = xq.detach().requires_grad_(True)
+    y = RMSNormModelFunction.apply(xg, w.to(DEV), 1e-6, d)
+    assert y.shape == xq.shape and y.stride() == xq.stride()          # same layout as the input view
+    y.backward(dy_base.to(DEV).transpose(1, 2))
+    yo, _, _ = O.rmsnorm_forward(base, w, 1e-6)
+    dxo, dwo = O.rmsnorm_backward(dy_base, base, w, 1e-6)
+    assert_bf16_close(y.transpose(1, 2), yo, "y")
+    assert_bf16_close(xg.grad.transpose(1, 2), dxo, "dx")
+    # identical bits to the contiguous path
+    y2 = ops.rmsnorm_forward(base.to(DEV), w.to(DEV), 1e-6)
+    assert torch.equal(y.transpose(1, 2), y2)
+    dx2, dw2 = ops.rmsnorm_backward(dy_base.to(DEV), base.to(DEV), w.to(DEV), 1e-6)
+    assert torch.equal(xg.grad.transpose(1, 2), dx2)
+    assert_grad_close(dw2, dwo, b * s * h, "dweight")
+    # a strided slice is not dense: falls back to a contiguous copy and still matches
+    xs = base.to(DEV)[:, ::2]
+    assert ops.memory_order_view(xs)[0] is None
+    assert_bf16_close(ops.rmsnorm_forward(xs, w.to(DEV), 1e-6), O.rmsnorm_forward(base[:, ::2], w, 1e-6)[0], "strided")
+
+
 def test_argument_errors():
     from teletron_amd import AdaLNModelFunction, RMSNormModelFunction, cabi, ops
     x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
