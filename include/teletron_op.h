@@ -147,7 +147,7 @@ TT_API int tt_reduce_partials(float* out0, float* out1, const void* workspace,
  * freqs is fp32 [seq_len][head_dim / 2][2] = (cos, sin) for position and complex index inside a
  * head (the reference's complex freqs[s, 1, head_dim / 2] viewed as real); row r uses position
  * r % seq_len, every head of a row the same table.  Backward multiplies dy by the conjugate and
- * continues as tt_rmsnorm_backward.  Requires cols % head_dim == 0, head_dim % 8 == 0,
+ * continues as tt_rmsnorm_backward.  Requires cols % head_dim == 0, head_dim % 8 == 0, head_dim <= 256,
  * cols > 256, 16-byte aligned tensors (TT_ERR_UNSUPPORTED otherwise).  Workspace as for
  * tt_rmsnorm_backward.  No counterpart in teletron_op.
  */

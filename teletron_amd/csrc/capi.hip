@@ -255,7 +255,8 @@ bool vector_path(int64_t cols, std::initializer_list<const void*> ptrs) {
 
 int check_rope(const Rope& rope, int64_t cols) {
   if (!rope.freqs || rope.head_dim <= 0 || rope.seq_len <= 0) return TT_ERR_INVALID_ARGUMENT;
-  if (rope.head_dim % kPack != 0 || cols % rope.head_dim != 0 || !aligned16(rope.freqs)) return TT_ERR_UNSUPPORTED;
+  if (rope.head_dim % kPack != 0 || rope.head_dim > 256 || cols % rope.head_dim != 0 || !aligned16(rope.freqs))
+    return TT_ERR_UNSUPPORTED;
   return TT_OK;
 }
 

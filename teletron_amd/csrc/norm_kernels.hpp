@@ -158,8 +158,14 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   // issued before the arithmetic of the current one, so every wave keeps a tile
   // in flight while it computes.
   u32x4 raw[R][P];
-  float fr[ROPE ? R : 1][ROPE ? P : 1][8];   // (cos, sin) of the packs being fetched
+  // ROPE: the (cos, sin) table of a row (head_dim floats, at most 256) is fetched once per row
+  // group by the first head_dim/4 lanes of its first wave, prefetched like the row itself, and
+  // handed to the other lanes through LDS: it is written before the barrier of the row
+  // reduction and read after it, two buffers alternating from tile to tile.
+  __shared__ __attribute__((aligned(16))) float ftab[ROPE ? 2 : 1][ROPE ? Q : 1][ROPE ? R : 1][ROPE ? 256 : 4];
+  f32x4 fq[R];
   int fcol[P];                               // column inside its head
+  const bool floader = ROPE && w == 0 && lane * 4 < a.head_dim;
   // Position of the first row of the tile that fetch() takes next, kept incrementally:
   // tiles are fetched in the order blockIdx.x, blockIdx.x + gridDim.x, ...
   int64_t fpos = 0, fstep = 0;
@@ -171,12 +177,14 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   }
   auto fetch = [&](int64_t t) {
     const int64_t r0 = t * (Q * R) + q * R;
-    int64_t pos[R];
     if constexpr (ROPE) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        pos[r] = fpos + r;
-        while (pos[r] >= a.seq_len) pos[r] -= a.seq_len;
+        int64_t pos = fpos + r;
+        while (pos >= a.seq_len) pos -= a.seq_len;
+        fq[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (floader && r0 + r < S)
+          fq[r] = *reinterpret_cast<const f32x4*>(a.freqs + (size_t)(pos * a.head_dim + lane * 4));
       }
       fpos += fstep;
       if (fpos >= a.seq_len) fpos -= a.seq_len;
@@ -186,22 +194,15 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
 #pragma unroll
       for (int p = 0; p < P; ++p) {
         raw[r][p] = u32x4{0, 0, 0, 0};
-        if constexpr (ROPE) {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) fr[r][p][j] = 0.f;
-        }
-        if (r0 + r < S && act[p]) {
-          raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
-          if constexpr (ROPE)
-            load_freq8(a.freqs, (size_t)(pos[r] * a.head_dim + fcol[p]), fr[r][p]);
-        }
+        if (r0 + r < S && act[p]) raw[r][p] = load_stream(a.x, (size_t)((b * S + r0 + r) * C + col[p]));
       }
   };
 
   unsigned phase = 0;
+  unsigned tpar = 0;
   int64_t tile = blockIdx.x;
   if (PF && tile < a.n_tiles) fetch(tile);
-  for (; tile < a.n_tiles; tile += gridDim.x) {
+  for (; tile < a.n_tiles; tile += gridDim.x, tpar ^= 1u) {
     const int64_t row0 = tile * (Q * R) + q * R;
     float xf[R][P][8];
     bool rv[R];
@@ -212,14 +213,11 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
 #pragma unroll
       for (int p = 0; p < P; ++p) unpack8(raw[r][p], xf[r][p]);
     }
-    float fc[ROPE ? R : 1][ROPE ? P : 1][8];
     if constexpr (ROPE) {
+      if (floader) {
 #pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int p = 0; p < P; ++p)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) fc[r][p][j] = fr[r][p][j];
+        for (int r = 0; r < R; ++r) *reinterpret_cast<f32x4*>(&ftab[tpar][q][r][lane * 4]) = fq[r];
+      }
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 
@@ -279,7 +277,14 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
               n[j] = xh;
               o[j] = ADALN ? fmaf(xh, g[p][j], sh[p][j]) : xh * g[p][j];
             }
-            if constexpr (ROPE) rope_rotate(o, fc[r][p]);
+            if constexpr (ROPE) {
+              float fc[8];
+              const f32x4* ft = reinterpret_cast<const f32x4*>(&ftab[tpar][q][r][fcol[p]]);
+              const f32x4 f0 = ft[0], f1 = ft[1];
+              fc[0] = f0[0]; fc[1] = f0[1]; fc[2] = f0[2]; fc[3] = f0[3];
+              fc[4] = f1[0]; fc[5] = f1[1]; fc[6] = f1[2]; fc[7] = f1[3];
+              rope_rotate(o, fc);
+            }
             store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
             if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col[p]), pack8(n));
           }
