@@ -167,6 +167,25 @@ size_t workspace_bound(int n_acc, int64_t rows, int64_t cols, int64_t rows_per_b
   return (size_t)n_batches * gx * n_acc * cols * sizeof(float);
 }
 
+// What the backward entry points of `kind` need for this shape: the partial sums of the plan they
+// will actually launch (the larger of the two backward contracts).  Falls back to the
+// plan-independent bound when a plan cannot be made here or a tuning override is active.
+size_t workspace_for(int kind, int n_acc, int64_t rows, int64_t cols, int64_t rows_per_batch) {
+  const size_t bound = workspace_bound(n_acc, rows, cols, rows_per_batch);
+  if (bound == 0 || cols % kPack != 0) return bound;
+  if (g_wgs_per_cu_override.load() > 0 || g_grid_override.load() > 0) return bound;
+  Plan p;
+  if (make_plan(kind, kBwd, rows, cols, rows_per_batch, &p) != TT_OK) return bound;
+  size_t need = partial_bytes(p, n_acc, cols);
+  if (kind != kGateKind && rows_per_batch == rows) {
+    Plan ps;
+    if (make_plan(kind, kBwdSaved, rows, cols, rows, &ps) != TT_OK) return bound;
+    const size_t ns = partial_bytes(ps, n_acc, cols);
+    if (ns > need) need = ns;
+  }
+  return need < 16 ? 16 : need;
+}
+
 template <typename Args>
 int launch(const Plan& p, Args& args, void* stream) {
   void* kargs[] = {&args};
@@ -386,10 +405,10 @@ int tt_rmsnorm_forward(void* y, const void* x, const void* weight, float* rstd,
 }
 
 size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch) {
-  return workspace_bound(2, rows, cols, rows_per_batch);
+  return workspace_for(kAdaLN, 2, rows, cols, rows_per_batch);
 }
 size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
-  return workspace_bound(1, rows, cols, rows);
+  return workspace_for(kRMS, 1, rows, cols, rows);
 }
 
 int tt_adaln_backward_partials(void* dx, const void* dy, const void* x, const void* scale,
@@ -476,7 +495,7 @@ int tt_gate_residual_forward(void* out, const void* x, const void* gate, const v
 }
 
 size_t tt_gate_residual_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch) {
-  return cols % kPack == 0 ? workspace_bound(1, rows, cols, rows_per_batch) : 0;
+  return cols % kPack == 0 ? workspace_for(kGateKind, 1, rows, cols, rows_per_batch) : 0;
 }
 
 int tt_gate_residual_backward(void* dresidual, float* dgate, const void* dout, const void* gate,
