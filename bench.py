@@ -46,7 +46,8 @@ def parse_args():
     ap.add_argument("--workload", default="adaln_wan14b")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
-    ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched",
+    ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched,"
+                                      "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
@@ -64,7 +65,8 @@ class GpuWorkload:
         self.lib = cabi.load()
         dev = torch.device("cuda:0")
         self.rows, self.cols = w.rows, w.cols
-        self.nb = w.param_shape[0] if w.op in ("adaln", "gate") else 1
+        self.ref = w.contract == "reference"
+        self.nb = w.param_shape[0] if w.op in ("adaln", "gate") and not self.ref else 1
         self.rpb = self.rows // self.nb
         g = torch.Generator(device=dev).manual_seed(seed)
         bf = torch.bfloat16
@@ -77,6 +79,10 @@ class GpuWorkload:
             s = {"x": randn(self.rows, self.cols), "dy": randn(self.rows, self.cols),
                  "y": torch.empty(self.rows, self.cols, dtype=bf, device=dev),
                  "dx": torch.empty(self.rows, self.cols, dtype=bf, device=dev)}
+            if self.ref:
+                s["rstd"] = torch.empty(self.rows, dtype=torch.float32, device=dev)
+                if w.op == "adaln":
+                    s["x_norm"] = torch.empty(self.rows, self.cols, dtype=bf, device=dev)
             self.sets.append(s)
         if w.op == "rope":
             self.p0 = randn(self.cols, scale=0.1, offset=1.0)              # gamma
@@ -101,14 +107,22 @@ class GpuWorkload:
             self.n_acc = 1
             ws_bytes = self.lib.tt_rmsnorm_backward_workspace_bytes(self.rows, self.cols)
         self.ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-        self.g0 = torch.empty(self.nb, self.cols, dtype=torch.float32, device=dev)
-        self.g1 = torch.empty(self.nb, self.cols, dtype=torch.float32, device=dev)
+        gdt = bf if self.ref else torch.float32
+        self.g0 = torch.empty(self.nb, self.cols, dtype=gdt, device=dev)
+        self.g1 = torch.empty(self.nb, self.cols, dtype=gdt, device=dev)
         self.n_partials = ctypes.c_int(0)
         self.stream = torch.cuda.current_stream().cuda_stream
 
     def fwd(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "rope":
+        if self.ref and self.w.op == "adaln":
+            self.cabi.call("tt_launch_adaln_forward", s["y"].data_ptr(), s["x_norm"].data_ptr(), s["x"].data_ptr(),
+                           self.p0.data_ptr(), self.p1.data_ptr(), self.rows, self.cols, self.w.eps,
+                           s["rstd"].data_ptr(), self.stream)
+        elif self.ref:
+            self.cabi.call("tt_launch_rms_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
+                           self.rows, self.cols, self.w.eps, s["rstd"].data_ptr(), self.stream)
+        elif self.w.op == "rope":
             self.cabi.call("tt_rmsnorm_rope_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
                            self.p1.data_ptr(), None, self.rows, self.cols, self.w.head_dim, self.w.shape[-2],
                            self.w.eps, self.stream)
@@ -124,7 +138,15 @@ class GpuWorkload:
 
     def bwd_partials(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.w.op == "rope":          # one entry point: streaming kernel + reduction of its partials
+        if self.ref and self.w.op == "adaln":   # one entry point: streaming kernel + reduction of its partials
+            self.cabi.call("tt_launch_adaln_backward", s["dx"].data_ptr(), self.g0.data_ptr(), self.g1.data_ptr(),
+                           s["dy"].data_ptr(), s["x_norm"].data_ptr(), self.p0.data_ptr(), s["rstd"].data_ptr(),
+                           self.rows, self.cols, self.ws.data_ptr(), self.ws.numel(), self.stream)
+        elif self.ref:
+            self.cabi.call("tt_launch_rms_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
+                           s["y"].data_ptr(), self.p0.data_ptr(), s["rstd"].data_ptr(), self.rows, self.cols,
+                           self.ws.data_ptr(), self.ws.numel(), self.stream)
+        elif self.w.op == "rope":          # one entry point: streaming kernel + reduction of its partials
             self.cabi.call("tt_rmsnorm_rope_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
                            s["x"].data_ptr(), self.p0.data_ptr(), self.p1.data_ptr(), self.ws.data_ptr(),
                            self.ws.numel(), self.rows, self.cols, self.w.head_dim, self.w.shape[-2], self.w.eps,
@@ -143,10 +165,30 @@ class GpuWorkload:
                            self.rows, self.cols, self.w.eps, self.stream)
 
     def reduce(self):
-        if self.w.op in ("gate", "rope"):
+        if self.w.op in ("gate", "rope") or self.ref:
             return
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
+
+    def stream_ceiling(self, iters=12):
+        """Bare streams over this workload's own buffers (no arithmetic, same load/store policy):
+        GB/s of one-read-one-write (x -> y) and two-reads-one-write (x ^ dy -> dx) traffic."""
+        torch = self.torch
+        nbytes = self.rows * self.cols * 2
+
+        def timed(two):
+            ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters + 3)]
+            for i, e in enumerate(ev):
+                s = self.sets[i % len(self.sets)]
+                e[0].record()
+                self.cabi.call("tt_stream_probe", (s["dx"] if two else s["y"]).data_ptr(), s["x"].data_ptr(),
+                               s["dy"].data_ptr() if two else None, nbytes, self.stream)
+                e[1].record()
+            torch.cuda.synchronize()
+            t = statistics.median(e[0].elapsed_time(e[1]) for e in ev[3:]) * 1e-3
+            return (3 if two else 2) * nbytes / t / 1e9
+
+        return {"copy": timed(False), "two_reads_one_write": timed(True)}
 
     def run(self, steps, warmup):
         """Returns wall seconds per step and per-kernel mean microseconds from HIP events."""
@@ -216,7 +258,7 @@ def cpu_baseline(w, seconds):
                       f"{t['x'].numel() // w.cols / med:.3e} rows/s, {per_elt:.0f} B/element"}
 
 
-def measure(w, steps, warmup):
+def measure(w, steps, warmup, ceiling=False):
     g = GpuWorkload(w)
     wall, k = g.run(steps, warmup)
     bytes_step = w.algorithmic_bytes("fwd+bwd")
@@ -230,6 +272,8 @@ def measure(w, steps, warmup):
         "bwd_gbps": w.algorithmic_bytes("bwd") / mean(k["bwd"]) / 1e3,
         "n_partials": g.n_partials.value,
     }
+    if ceiling:
+        res["ceiling"] = g.stream_ceiling()
     del g   # the caching allocator keeps the blocks: later workloads reuse them instead of fresh driver memory
     return res
 
@@ -246,7 +290,7 @@ def main():
         print("bench.py needs a GPU: the HIP kernels have no CPU fallback.", file=sys.stderr)
         return 2
     w = WORKLOADS[args.workload]
-    r = measure(w, args.steps, args.warmup)
+    r = measure(w, args.steps, args.warmup, ceiling=True)
     mt = MEASURED_TRAFFIC_BYTES.get(w.name)
     traffic = mt["bwd"] if mt and mt["n_partials"] == r["n_partials"] else None
     out = {
@@ -268,6 +312,14 @@ def main():
                                         "frac": round(r["fwd_gbps"] / HBM_PEAK_GBPS, 4),
                                         "algorithmic_bytes_per_launch": w.algorithmic_bytes("fwd")}},
     }
+    # The machine's own streaming ceiling, measured in this run on the same buffers: the forward
+    # kernel is 1 read : 1 write traffic, the backward kernel 2 reads : 1 write.
+    c = r["ceiling"]
+    out["stream_ceiling"] = {
+        "unit": "GB/s", "copy": round(c["copy"], 1), "two_reads_one_write": round(c["two_reads_one_write"], 1),
+        "forward_frac_of_copy": round(r["fwd_gbps"] / c["copy"], 4),
+        "backward_frac_of_two_reads_one_write": round(r["bwd_gbps"] / c["two_reads_one_write"], 4),
+        "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers"}
     also = {}
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         wa = WORKLOADS[name]

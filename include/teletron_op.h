@@ -179,6 +179,15 @@ TT_API int tt_gate_residual_backward(void* dresidual, float* dgate, const void* 
                                      int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream);
 TT_API size_t tt_gate_residual_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch);
 
+/* ------------------------------------------------------------------ bare streaming probe
+ * Measurement aid without a counterpart in the reference: out[i] = a[i] (b == NULL) or
+ * a[i] ^ b[i] over `bytes` bytes, with the load/store policy of the kernels above, one
+ * workgroup per compute unit and no arithmetic.  A benchmark runs it on the same buffers to report
+ * what plain one-read-one-write and two-reads-one-write traffic reaches on the machine at hand,
+ * next to the published HBM peak.  bytes % 16 == 0 and 16-byte aligned pointers
+ * (TT_ERR_UNSUPPORTED otherwise); bytes == 0 is a no-op. */
+TT_API int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void* stream);
+
 /* ------------------------------------------------------------------ reference-compatible contract
  * Argument for argument the launchers the reference's pybind glue calls, plus a trailing
  * stream (the reference launches on the legacy default stream) and, for backward, the

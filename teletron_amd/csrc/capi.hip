@@ -9,6 +9,7 @@
 
 #include "generic_kernels.hpp"
 #include "kernel_table.hpp"
+#include "probe_kernels.hpp"
 
 namespace tt {
 namespace {
@@ -182,6 +183,13 @@ size_t workspace_for(int kind, int n_acc, int64_t rows, int64_t cols, int64_t ro
     if (make_plan(kind, kBwdSaved, rows, cols, rows, &ps) != TT_OK) return bound;
     const size_t ns = partial_bytes(ps, n_acc, cols);
     if (ns > need) need = ns;
+  }
+  if (kind == kRMS && cols / kPack > kNarrowMaxPacks) {   // tt_rmsnorm_rope_backward shares this size query
+    Plan pr;
+    if (make_plan(kRMS, kBwd, rows, cols, rows, &pr, true) == TT_OK) {
+      const size_t nr = partial_bytes(pr, n_acc, cols);
+      if (nr > need) need = nr;
+    }
   }
   return need < 16 ? 16 : need;
 }
@@ -514,6 +522,24 @@ int tt_gate_residual_backward(void* dresidual, float* dgate, const void* dout, c
   rc = launch(p, a, stream);
   if (rc != TT_OK) return rc;
   return reduce(dgate, nullptr, workspace, (int)(rows / rows_per_batch), p.grid_x, 1, cols, false, stream);
+}
+
+// ---------------------------------------------------------------- bare streaming probe
+int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void* stream) {
+  if (bytes == 0) return TT_OK;
+  if (!out || !a) return TT_ERR_INVALID_ARGUMENT;
+  if (bytes % 16 != 0 || !aligned16(out) || !aligned16(a) || !aligned16(b)) return TT_ERR_UNSUPPORTED;
+  int cus = 0;
+  const int rc = current_device_cus(&cus);
+  if (rc != TT_OK) return rc;
+  const size_t n = bytes / 16;
+  const size_t want = (n + kProbeThreads - 1) / kProbeThreads;
+  const dim3 grid((unsigned)(want < (size_t)cus ? want : (size_t)cus));   // one workgroup per CU
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (b) hipLaunchKernelGGL((stream_probe<true, 1>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  else   hipLaunchKernelGGL((stream_probe<false, 2>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TT_OK : hip_fail(e);
 }
 
 // ---------------------------------------------------------------- reference-compatible contract

@@ -21,6 +21,7 @@ class Workload:
     eps: float = 1e-6
     note: str = ""
     head_dim: int = 0            # "rope" only
+    contract: str = "native"     # "native" (saves x) | "reference" (tt_launch_*: saves x_norm / y and rstd)
 
     @property
     def cols(self) -> int:
@@ -54,6 +55,12 @@ class Workload:
             bwd = 6 * e + n_param * 2 + n_param * 4
             return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
         n_vec = 2 if self.op == "adaln" else 1
+        if self.contract == "reference":
+            # forward also stores rstd (fp32 per row) and, for AdaLN, x_norm; backward reads the saved
+            # activation + rstd and returns bf16 parameter gradients
+            fwd = (6 if self.op == "adaln" else 4) * e + n_vec * n_param * 2 + self.rows * 4
+            bwd = 6 * e + n_param * 2 + n_vec * n_param * 2 + self.rows * 4
+            return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
         fwd = 4 * e + n_vec * n_param * 2
         bwd = 6 * e + n_param * 2 + n_vec * n_param * 4
         return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
@@ -68,6 +75,10 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
     Workload("adaln_odd", "adaln", (3, 5000, 1000), (3, 1, 1000), note="125 packs per row: ragged wave tail"),
     Workload("rmsnorm_rope_wan14b", "rope", (1, 75600, 5120), (5120,), head_dim=128,
              note="Wan2.1-14B QK-norm + rotary embedding, 40 heads of 128"),
+    Workload("adaln_hunyuan_reference_contract", "adaln", (1, 118800, 3072), (3072,), contract="reference",
+             note="the reference's own AdaLN width, through its launcher signatures"),
+    Workload("rmsnorm_hunyuan_head_reference_contract", "rmsnorm", (1, 118800, 24, 128), (128,), contract="reference",
+             note="the reference's own RMSNorm width, through its launcher signatures"),
     Workload("gate_wan14b", "gate", (1, 75600, 5120), (1, 1, 5120), note="gated residual add after each AdaLN site"),
 ]}
 

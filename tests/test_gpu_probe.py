@@ -1,0 +1,35 @@
+"""The bare streaming probe (tt_stream_probe) moves bytes exactly: bit-exact copy / xor, ragged
+sizes included, and refuses what it documents as unsupported."""
+import pytest
+import torch
+
+from test_gpu_parity import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n_packs", [1, 63, 512, 513, 256 * 512 * 2 + 77, 3_000_001])
+def test_stream_probe_copy_and_xor(n_packs):
+    from teletron_amd import cabi
+    g = torch.Generator().manual_seed(n_packs)
+    a = torch.randint(-2**31, 2**31 - 1, (n_packs * 4 + 4,), generator=g, dtype=torch.int32).to(DEV)
+    b = torch.randint(-2**31, 2**31 - 1, (n_packs * 4 + 4,), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.full_like(a, 7)
+    stream = torch.cuda.current_stream().cuda_stream
+    cabi.call("tt_stream_probe", out.data_ptr(), a.data_ptr(), None, n_packs * 16, stream)
+    assert torch.equal(out[:n_packs * 4], a[:n_packs * 4])
+    assert torch.all(out[n_packs * 4:] == 7)           # nothing past the end is touched
+    cabi.call("tt_stream_probe", out.data_ptr(), a.data_ptr(), b.data_ptr(), n_packs * 16, stream)
+    assert torch.equal(out[:n_packs * 4], a[:n_packs * 4] ^ b[:n_packs * 4])
+    assert torch.all(out[n_packs * 4:] == 7)
+
+
+def test_stream_probe_errors():
+    from teletron_amd import cabi
+    lib = cabi.load()
+    a = torch.zeros(64, dtype=torch.int32, device=DEV)
+    out = torch.zeros_like(a)
+    assert lib.tt_stream_probe(out.data_ptr(), a.data_ptr(), None, 0, None) == cabi.TT_OK
+    assert lib.tt_stream_probe(None, a.data_ptr(), None, 64, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_stream_probe(out.data_ptr(), a.data_ptr(), None, 24, None) == cabi.TT_ERR_UNSUPPORTED
+    assert lib.tt_stream_probe(out.data_ptr() + 4, a.data_ptr(), None, 64, None) == cabi.TT_ERR_UNSUPPORTED
