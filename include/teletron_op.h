@@ -179,6 +179,40 @@ TT_API int tt_gate_residual_backward(void* dresidual, float* dgate, const void* 
                                      int64_t rows, int64_t cols, int64_t rows_per_batch, void* stream);
 TT_API size_t tt_gate_residual_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch);
 
+/* ------------------------------------------------------------------ residual update + LayerNorm
+ * The residual update of a DiT block fused with the normalisation that reads its result
+ * (teletron/models/wan/wan_model.py:239-241: `x = self.gate(x, gate_msa, attn_output)`,
+ * `x = x + self.cross_attn(self.norm3(x), context)`, `modulate(self.norm2(x), shift_mlp, scale_mlp)`):
+ *
+ *   s = x + gate * r      (gate != NULL)      or      s = x + r
+ *   y = LayerNorm(s) * (1 + scale) + shift    (affine == 0: AdaLN modulation)
+ *   y = LayerNorm(s) * scale + shift          (affine != 0: nn.LayerNorm weight / bias, wan_model.py:224)
+ *
+ * s is rounded to bf16 and it is the rounded value that is normalised, as in the unfused
+ * sequence.  gate holds n_gate vectors of cols elements and scale / shift n_param vectors each,
+ * where a count is 1 (shared by all batches) or rows / rows_per_batch (one per batch).
+ * Vector path only: cols % 8 == 0, cols > 256, 16-byte aligned tensors (TT_ERR_UNSUPPORTED
+ * otherwise; callers then run the two operations separately).  mean / rstd: optional [rows] fp32.
+ *
+ * Backward receives dy (gradient of y) and ds_in (gradient reaching s from its other consumers;
+ * NULL = none) and the saved s:
+ *   dx = ds_in + dLayerNorm(dy)      gradient of x, and of r when there is no gate
+ *   dr = gate * dx, dgate = sum over rows of dx * r         (gate != NULL)
+ *   dscale = sum over rows of dy * x_hat, dshift = sum over rows of dy
+ * dscale, dshift, dgate: fp32 [rows / rows_per_batch, cols], one vector per batch even where the
+ * parameter is shared (the caller adds the batches of a shared parameter).  Deterministic. */
+TT_API int tt_residual_norm_forward(void* s, void* y, const void* x, const void* r,
+                                    const void* gate, int64_t n_gate,
+                                    const void* scale, const void* shift, int64_t n_param, int affine,
+                                    float* mean, float* rstd,
+                                    int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream);
+TT_API int tt_residual_norm_backward(void* dx, void* dr, float* dscale, float* dshift, float* dgate,
+                                     const void* dy, const void* ds_in, const void* s, const void* r,
+                                     const void* gate, int64_t n_gate, const void* scale, int64_t n_param, int affine,
+                                     void* workspace, size_t workspace_bytes,
+                                     int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream);
+TT_API size_t tt_residual_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch, int gated);
+
 /* ------------------------------------------------------------------ bare streaming probe
  * Measurement aid without a counterpart in the reference: out[i] = a[i] (b == NULL) or
  * a[i] ^ b[i] over `bytes` bytes, with the load/store policy of the kernels above, one

@@ -225,6 +225,40 @@ def gate_residual_backward(dout, gate, residual, n_batches: int = 1):
     return _f64(dout), (d * r).sum(dim=1), (d * g).reshape(dout.shape)
 
 
+# --------------------------------------------------------------------------- residual update + LayerNorm
+def residual_norm_forward(x, residual, gate, scale, shift, eps: float, n_batches: int = 1, affine: bool = False,
+                          round_s: bool = True):
+    """The residual update of a DiT block followed by the normalisation that reads it
+    (teletron/models/wan/wan_model.py:239-241):  s = x + gate * residual (gate None: x + residual),
+    y = LayerNorm(s) * (1 + scale) + shift, or with ``affine`` LayerNorm(s) * scale + shift
+    (nn.LayerNorm weight / bias, wan_model.py:224).  The residual stream is a bf16 tensor, so with
+    ``round_s`` the normalisation reads s rounded to bf16.  Returns ``(s, y)`` in float64."""
+    c = x.shape[-1]
+    if gate is None:
+        s = _f64(x) + _f64(residual)
+    else:
+        s = gate_residual_forward(x, gate, residual, n_batches)
+    if round_s:
+        s = s.to(torch.bfloat16).to(F64)
+    sc = _param(scale, n_batches, c) - (1.0 if affine else 0.0)
+    y = adaln_forward(s, sc, shift, eps, n_batches)[0]
+    return s, y
+
+
+def residual_norm_backward(dy, ds_in, s, residual, gate, scale, eps: float, n_batches: int = 1, affine: bool = False):
+    """Gradients of the above from the saved s: ds = ds_in + dLayerNorm(dy) is the gradient of x (and of
+    the residual when there is no gate); with a gate dresidual = gate * ds and dgate = sum_rows ds * residual.
+    Returns ``(ds, dresidual, dscale[B,C], dshift[B,C], dgate[B,C] or None)``."""
+    c = s.shape[-1]
+    sc = _param(scale, n_batches, c) - (1.0 if affine else 0.0)
+    dn, dscale, dshift = adaln_backward(dy, s, sc, eps, n_batches)
+    ds = dn if ds_in is None else dn + _f64(ds_in)
+    if gate is None:
+        return ds, ds, dscale, dshift, None
+    _, dgate, dres = gate_residual_backward(ds, gate, residual, n_batches)
+    return ds, dres, dscale, dshift, dgate
+
+
 # --------------------------------------------------------------------------- chunked variants
 def adaln_backward_param_grads_chunked(dy, x, eps: float, n_batches: int = 1, chunk_rows: int = 4096):
     """dscale / dshift only, streamed over row chunks so that full-size shapes

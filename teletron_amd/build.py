@@ -20,7 +20,8 @@ OBJ_DIR = CSRC / "build"
 LIB_PATH = PKG_DIR / "libteletron_op.so"
 
 HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_bwd.hip", "adaln_bwd_saved.hip",
-               "rms_fwd.hip", "rms_bwd.hip", "rms_bwd_saved.hip", "rms_rope.hip", "gate.hip"]
+               "rms_fwd.hip", "rms_bwd.hip", "rms_bwd_saved.hip", "rms_rope.hip", "gate.hip",
+               "resnorm_plain.hip", "resnorm_gated.hip"]
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form
 # v_pk_{add,mul,fma}_f32 from the scalar float code of these kernels.

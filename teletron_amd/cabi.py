@@ -60,6 +60,14 @@ PROTOTYPES = {
     "tt_gate_residual_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                           c_int64, c_int64, c_int64, c_void_p]),
     "tt_gate_residual_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "tt_residual_norm_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                         c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p,
+                                         c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_residual_norm_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_int64, c_void_p, c_int64, c_int,
+                                          c_void_p, c_size_t, c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_residual_norm_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "tt_stream_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tt_launch_adaln_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int64, c_double, c_void_p, c_void_p]),

@@ -87,7 +87,9 @@ constexpr int kGateKind = 2;   // third op family next to kAdaLN / kRMS
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
 constexpr int kMaxWgsPerCu = 8;
 
-int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan, bool rope = false) {
+// `res`: 0, or the residual + LayerNorm fusion: 1 plain, 2 gated (wide rows, kFwd / kBwd only).
+int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan, bool rope = false,
+              int res = 0) {
   if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0)
     return TT_ERR_INVALID_ARGUMENT;
   if (cols > TT_MAX_COLS) return TT_ERR_UNSUPPORTED;
@@ -99,7 +101,10 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   const int slots = narrow ? kNarrowL[idx] : 64 * kWideW[idx] * kWideP[idx];
   const bool full = (slots == packs);
   KernelInfo k;
-  if (rope) {
+  if (res) {
+    if (narrow || kind != kAdaLN || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
+    k = res == 2 ? resnorm_gated_kernel(dir == kBwd, idx, full) : resnorm_plain_kernel(dir == kBwd, idx, full);
+  } else if (rope) {
     if (narrow || kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
     k = rms_rope_kernel(dir == kBwd, idx, full);
   } else if (kind == kAdaLN)
@@ -127,7 +132,7 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   if (!cache_resident) {
     const int per_wg = (k.threads / kWave) * k.lane_loads;
     // two streamed inputs (backward kernels, both gate kernels) or one (normalisation forward)
-    const int target = (dir == kFwd && kind != kGateKind) ? kFwdLoadsPerCu : kBwdLoadsPerCu;
+    const int target = (dir == kFwd && kind != kGateKind && !res) ? kFwdLoadsPerCu : kBwdLoadsPerCu;
     int want = (2 * target + per_wg) / (2 * per_wg);
     if (want < 1) want = 1;
     if (want < per_cu) per_cu = want;
@@ -358,17 +363,18 @@ int backward_saved_partials(int kind, void* dx, const void* dy, const void* xs, 
 }
 
 int reduce(void* out0, void* out1, const void* workspace, int n_batches, int n_partials, int n_acc,
-           int64_t cols, bool out_bf16, void* stream) {
+           int64_t cols, bool out_bf16, void* stream, void* out2 = nullptr) {
   if (n_batches == 0) return TT_OK;
   if (!out0 || !workspace || n_batches < 0 || n_batches > 65535 || n_partials <= 0 || cols <= 0 ||
-      cols > TT_MAX_COLS || (n_acc != 1 && n_acc != 2) || (n_acc == 2 && !out1))
+      cols > TT_MAX_COLS || n_acc < 1 || n_acc > 3 || (n_acc >= 2 && !out1) || (n_acc == 3 && !out2))
     return TT_ERR_INVALID_ARGUMENT;
   const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)n_batches, 1);
   const float* ws = static_cast<const float*>(workspace);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int bf = out_bf16 ? 1 : 0;
-  if (n_acc == 2) hipLaunchKernelGGL(reduce_partials<2>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols, bf);
-  else            hipLaunchKernelGGL(reduce_partials<1>, grid, dim3(1024), 0, s, out0, out1, ws, n_partials, (int)cols, bf);
+  if (n_acc == 3)      hipLaunchKernelGGL(reduce_partials<3>, grid, dim3(1024), 0, s, out0, out1, out2, ws, n_partials, (int)cols, bf);
+  else if (n_acc == 2) hipLaunchKernelGGL(reduce_partials<2>, grid, dim3(1024), 0, s, out0, out1, out2, ws, n_partials, (int)cols, bf);
+  else                 hipLaunchKernelGGL(reduce_partials<1>, grid, dim3(1024), 0, s, out0, out1, out2, ws, n_partials, (int)cols, bf);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return TT_OK;
@@ -522,6 +528,66 @@ int tt_gate_residual_backward(void* dresidual, float* dgate, const void* dout, c
   rc = launch(p, a, stream);
   if (rc != TT_OK) return rc;
   return reduce(dgate, nullptr, workspace, (int)(rows / rows_per_batch), p.grid_x, 1, cols, false, stream);
+}
+
+// ---------------------------------------------------------------- residual update + LayerNorm
+// scale / shift / gate hold either one vector for all batches or one per batch.
+static bool stride_ok(int64_t n_vectors, int64_t n_batches) { return n_vectors == 1 || n_vectors == n_batches; }
+
+int tt_residual_norm_forward(void* s, void* y, const void* x, const void* r, const void* gate, int64_t n_gate,
+                             const void* scale, const void* shift, int64_t n_param, int affine,
+                             float* mean, float* rstd, int64_t rows, int64_t cols, int64_t rows_per_batch,
+                             float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!s || !y || !x || !r || !scale || !shift) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {s, y, x, r, gate, scale, shift})) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kAdaLN, kFwd, rows, cols, rows_per_batch, &p, false, gate ? 2 : 1);
+  if (rc != TT_OK) return rc;
+  if (!stride_ok(n_param, p.n_batches) || (gate && !stride_ok(n_gate, p.n_batches))) return TT_ERR_INVALID_ARGUMENT;
+  ResFwdArgs a;
+  a.s = s; a.y = y; a.x = x; a.r = r; a.gate = gate; a.scale = scale; a.shift = shift; a.mean = mean; a.rstd = rstd;
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
+  a.gate_stride = n_gate == 1 ? 0 : cols; a.param_stride = n_param == 1 ? 0 : cols;
+  a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols; a.one = affine ? 0.f : 1.f;
+  return launch(p, a, stream);
+}
+
+size_t tt_residual_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch, int gated) {
+  if (rows <= 0 || cols <= 0 || cols % kPack != 0) return 0;
+  Plan p;
+  if (make_plan(kAdaLN, kBwd, rows, cols, rows_per_batch, &p, false, gated ? 2 : 1) != TT_OK) return 0;
+  if (g_wgs_per_cu_override.load() > 0 || g_grid_override.load() > 0)
+    return workspace_bound(gated ? 3 : 2, rows, cols, rows_per_batch);
+  const size_t need = partial_bytes(p, gated ? 3 : 2, cols);
+  return need < 16 ? 16 : need;
+}
+
+int tt_residual_norm_backward(void* dx, void* dr, float* dscale, float* dshift, float* dgate,
+                              const void* dy, const void* ds_in, const void* s, const void* r,
+                              const void* gate, int64_t n_gate, const void* scale, int64_t n_param, int affine,
+                              void* workspace, size_t workspace_bytes,
+                              int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
+  if (rows == 0) return TT_OK;
+  const bool gated = gate != nullptr;
+  if (!dx || !dscale || !dshift || !dy || !s || !scale) return TT_ERR_INVALID_ARGUMENT;
+  if (gated && (!dr || !dgate || !r)) return TT_ERR_INVALID_ARGUMENT;
+  if (!vector_path(cols, {dx, dr, dy, ds_in, s, r, gate, scale})) return TT_ERR_UNSUPPORTED;
+  Plan p;
+  int rc = make_plan(kAdaLN, kBwd, rows, cols, rows_per_batch, &p, false, gated ? 2 : 1);
+  if (rc != TT_OK) return rc;
+  if (!stride_ok(n_param, p.n_batches) || (gated && !stride_ok(n_gate, p.n_batches))) return TT_ERR_INVALID_ARGUMENT;
+  const int n_acc = gated ? 3 : 2;
+  if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;
+  ResBwdArgs a;
+  a.dx = dx; a.dr = dr; a.dy = dy; a.ds_in = ds_in; a.s = s; a.r = r; a.gate = gate; a.scale = scale;
+  a.partials = static_cast<float*>(workspace);
+  a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
+  a.gate_stride = n_gate == 1 ? 0 : cols; a.param_stride = n_param == 1 ? 0 : cols;
+  a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols; a.one = affine ? 0.f : 1.f;
+  rc = launch(p, a, stream);
+  if (rc != TT_OK) return rc;
+  return reduce(dscale, dshift, workspace, (int)p.n_batches, p.grid_x, n_acc, cols, false, stream, dgate);
 }
 
 // ---------------------------------------------------------------- bare streaming probe

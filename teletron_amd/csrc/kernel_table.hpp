@@ -5,6 +5,7 @@
 #pragma once
 #include "gate_kernels.hpp"
 #include "norm_kernels.hpp"
+#include "resnorm_kernels.hpp"
 
 namespace tt {
 
@@ -208,6 +209,47 @@ KernelInfo lookup_gate(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
+// Residual update fused with the following LayerNorm (wide rows only): forward streams two
+// inputs, backward three (four with a gate).
+constexpr int res_fwd_Q(int W, int P) {
+#ifdef TT_RES_FWD_Q
+  return TT_RES_FWD_Q * W > 16 ? 1 : TT_RES_FWD_Q;
+#else
+  return bwd_wide_Q(W, P);
+#endif
+}
+constexpr int res_bwd_Q(int W, int P, bool gated) {
+#ifdef TT_RES_BWD_Q
+  return TT_RES_BWD_Q * W > 16 ? 1 : TT_RES_BWD_Q;
+#else
+  int q = bwd_wide_Q(W, P);
+  while (q > 1 && W * q > 8) --q;   // three or four streamed inputs: at most 8 waves, 256 VGPRs per lane
+  return q;
+#endif
+}
+template <int W, int P, bool FULL, bool GATED>
+KernelInfo info_res_fwd() {
+  constexpr int R = 1, Q = res_fwd_Q(W, P);
+  return {reinterpret_cast<const void*>(&resnorm_fwd_wide<W, P, R, Q, FULL, GATED>), 64 * W * Q, Q * R, P * R};
+}
+template <int W, int P, bool FULL, bool GATED>
+KernelInfo info_res_bwd() {
+  constexpr int R = 1, Q = res_bwd_Q(W, P, GATED);
+  return {reinterpret_cast<const void*>(&resnorm_bwd_wide<W, P, R, Q, FULL, GATED>), 64 * W * Q, Q * R, P * R};
+}
+template <bool GATED>
+KernelInfo lookup_res(bool backward, int idx, bool full) {
+  switch (idx) {
+#define X(i, W, P)                                                                                        \
+  case i:                                                                                                 \
+    return backward ? (full ? info_res_bwd<W, P, true, GATED>() : info_res_bwd<W, P, false, GATED>())     \
+                    : (full ? info_res_fwd<W, P, true, GATED>() : info_res_fwd<W, P, false, GATED>());
+    TT_WIDE_LIST(X)
+#undef X
+  }
+  return {nullptr, 0, 0, 0};
+}
+
 template <int KIND>
 KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   if (narrow) {
@@ -226,7 +268,8 @@ KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
-// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, rms_rope.hip, gate.hip).
+// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, rms_rope.hip, gate.hip,
+// resnorm_plain.hip, resnorm_gated.hip).
 KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
@@ -236,5 +279,7 @@ KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_rope_kernel(bool backward, int idx, bool full);
 KernelInfo gate_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo gate_bwd_kernel(bool narrow, int idx, bool full);
+KernelInfo resnorm_plain_kernel(bool backward, int idx, bool full);
+KernelInfo resnorm_gated_kernel(bool backward, int idx, bool full);
 
 }  // namespace tt

@@ -997,7 +997,7 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_saved_narrow(const BwdSavedA
 // The output is fp32, or bf16 (rounded once) when out_bf16 is set.
 template <int NACC>
 __global__ __launch_bounds__(1024) void reduce_partials(void* __restrict__ out0, void* __restrict__ out1,
-                                                        const float* __restrict__ partials,
+                                                        void* __restrict__ out2, const float* __restrict__ partials,
                                                         int n_partials, int cols, int out_bf16) {
   __shared__ float fold[16][NACC][64];
   const int lane = threadIdx.x & 63;
@@ -1034,7 +1034,7 @@ __global__ __launch_bounds__(1024) void reduce_partials(void* __restrict__ out0,
     float t = fold[0][wave][lane];
 #pragma unroll
     for (int ww = 1; ww < 16; ++ww) t += fold[ww][wave][lane];
-    void* out = wave == 0 ? out0 : out1;
+    void* out = wave == 0 ? out0 : wave == 1 ? out1 : out2;
     const size_t idx = (size_t)b * cols + c;
     if (out_bf16) static_cast<uint16_t*>(out)[idx] = f32_to_bf16(t);
     else          static_cast<float*>(out)[idx] = t;

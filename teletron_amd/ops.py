@@ -268,3 +268,86 @@ def rmsnorm_rope_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tenso
                   weight.data_ptr(), freqs.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, head_dim, seq,
                   float(eps), _stream(x))
     return dx, dweight
+
+
+# --------------------------------------------------------------------------- residual update + LayerNorm
+RESIDUAL_NORM_MIN_COLS = 264     # the fused kernels cover rows of more than 256 elements
+
+
+def residual_norm_supported(x: torch.Tensor) -> bool:
+    """True where ``residual_norm_forward`` has a fused kernel: bf16 on a GPU, cols % 8 == 0, cols > 256."""
+    return (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == BF16 and x.dim() >= 1
+            and x.shape[-1] % 8 == 0 and RESIDUAL_NORM_MIN_COLS <= x.shape[-1] <= 32768)
+
+
+def _res_batches(rows: int, cols: int, gate: Optional[torch.Tensor], scale: torch.Tensor):
+    n_param = scale.numel() // cols
+    n_gate = gate.numel() // cols if gate is not None else 1
+    nb = max(n_param, n_gate)
+    _require(n_param in (1, nb) and n_gate in (1, nb), ValueError,
+             f"gate holds {n_gate} vectors and scale/shift {n_param}: each must be 1 or the number of batches")
+    _require(rows % nb == 0, ValueError, f"{nb} parameter vectors do not divide the {rows} rows of the input")
+    return nb, rows // nb, n_gate, n_param
+
+
+def residual_norm_forward(x: torch.Tensor, residual: torch.Tensor, gate: Optional[torch.Tensor],
+                          scale: torch.Tensor, shift: torch.Tensor, eps: float, affine: bool = False):
+    """s = x + gate * residual (gate None: x + residual); y = LayerNorm(s) * (1 + scale) + shift, or
+    LayerNorm(s) * scale + shift with ``affine`` (scale = weight, shift = bias).  Returns (s, y)."""
+    cols = x.shape[-1]
+    x = _check_act("x", x, cols)
+    residual = _check_act("residual", residual, cols)
+    _require(residual.numel() == x.numel() and residual.device == x.device, ValueError,
+             "residual must match x in size and device")
+    scale = _check_param("scale", scale, x, cols)
+    shift = _check_param("shift", shift, x, cols)
+    _require(scale.numel() == shift.numel(), ValueError, "scale and shift must have the same number of elements")
+    if gate is not None:
+        gate = _check_param("gate", gate, x, cols)
+    rows = x.numel() // cols
+    s, y = torch.empty_like(x), torch.empty_like(x)
+    if rows:
+        nb, rpb, n_gate, n_param = _res_batches(rows, cols, gate, scale)
+        with torch.cuda.device(x.device):
+            cabi.call("tt_residual_norm_forward", s.data_ptr(), y.data_ptr(), x.data_ptr(), residual.data_ptr(),
+                      _ptr(gate), n_gate, scale.data_ptr(), shift.data_ptr(), n_param, int(bool(affine)),
+                      None, None, rows, cols, rpb, float(eps), _stream(x))
+    return s, y
+
+
+def residual_norm_backward(dy: torch.Tensor, ds_in: Optional[torch.Tensor], s: torch.Tensor,
+                           residual: Optional[torch.Tensor], gate: Optional[torch.Tensor], scale: torch.Tensor,
+                           eps: float, affine: bool = False):
+    """Backward of ``residual_norm_forward`` from the saved ``s``.  ``ds_in`` is the gradient that
+    reaches ``s`` from its other consumers (None = none).  Returns
+    ``(dx, dresidual, dscale, dshift, dgate)``: dx / dresidual bf16 (the same tensor when there is
+    no gate), the parameter gradients fp32 ``[n_batches, C]`` (dgate None without a gate)."""
+    cols = s.shape[-1]
+    s = _check_act("s", s, cols)
+    dy = _check_act("dy", dy, cols)
+    _require(dy.numel() == s.numel() and dy.device == s.device, ValueError, "dy must match s in size and device")
+    if ds_in is not None:
+        ds_in = _check_act("ds_in", ds_in, cols)
+        _require(ds_in.numel() == s.numel() and ds_in.device == s.device, ValueError, "ds_in must match s")
+    scale = _check_param("scale", scale, s, cols)
+    if gate is not None:
+        gate = _check_param("gate", gate, s, cols)
+        residual = _check_act("residual", residual, cols)
+        _require(residual.numel() == s.numel() and residual.device == s.device, ValueError, "residual must match s")
+    rows = s.numel() // cols
+    nb, rpb, n_gate, n_param = _res_batches(rows, cols, gate, scale) if rows else (max(scale.numel() // cols, 1), 0, 1, 1)
+    dx = torch.empty_like(s)
+    dr = torch.empty_like(s) if gate is not None else dx
+    f32 = dict(dtype=torch.float32, device=s.device)
+    if rows == 0:
+        return dx, dr, torch.zeros(nb, cols, **f32), torch.zeros(nb, cols, **f32), \
+            (torch.zeros(nb, cols, **f32) if gate is not None else None)
+    dscale, dshift = torch.empty(nb, cols, **f32), torch.empty(nb, cols, **f32)
+    dgate = torch.empty(nb, cols, **f32) if gate is not None else None
+    with torch.cuda.device(s.device):
+        ws = _workspace(cabi.load().tt_residual_norm_backward_workspace_bytes(rows, cols, rpb, int(gate is not None)), 0, s)
+        cabi.call("tt_residual_norm_backward", dx.data_ptr(), _ptr(dr if gate is not None else None),
+                  dscale.data_ptr(), dshift.data_ptr(), _ptr(dgate), dy.data_ptr(), _ptr(ds_in), s.data_ptr(),
+                  _ptr(residual if gate is not None else None), _ptr(gate), n_gate, scale.data_ptr(), n_param,
+                  int(bool(affine)), ws.data_ptr(), ws.numel(), rows, cols, rpb, float(eps), _stream(s))
+    return dx, dr, dscale, dshift, dgate

@@ -263,6 +263,50 @@ def test_gate_residual_matches_autograd():
     torch.testing.assert_close(O.gate_residual_forward(x, torch.ones(nb, c), r, nb), (x + r).detach(), rtol=0, atol=1e-15)
 
 
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("affine", [False, True])
+def test_residual_norm_matches_autograd(gated, affine):
+    """The fused residual update + LayerNorm against torch's own layer_norm and autograd on the
+    unfused float64 expression, with gradients arriving at both outputs."""
+    nb, s, c, eps = 3, 7, 24, 1e-5
+    leaf = lambda *shape, seed, scale=1.0: rnd(*shape, seed=seed, scale=scale).requires_grad_(True)
+    x, r = leaf(nb, s, c, seed=70), leaf(nb, s, c, seed=71)
+    g = leaf(nb, 1, c, seed=72, scale=0.5) if gated else None
+    if affine:       # one weight / bias for all batches, as nn.LayerNorm(dim)
+        sc, sh = leaf(c, seed=73), leaf(c, seed=74)
+    else:            # per-sample modulation
+        sc, sh = leaf(nb, 1, c, seed=73, scale=0.3), leaf(nb, 1, c, seed=74, scale=0.3)
+    dy, ds_in = rnd(nb, s, c, seed=75), rnd(nb, s, c, seed=76)
+    st = x + (g * r if gated else r)
+    if affine:
+        yt = torch.nn.functional.layer_norm(st, (c,), sc, sh, eps)
+    else:
+        yt = torch.nn.functional.layer_norm(st, (c,), None, None, eps) * (1 + sc) + sh
+    (yt * dy).sum().add((st * ds_in).sum()).backward()
+    n_param = 1 if affine else nb
+    so, yo = O.residual_norm_forward(x, r, g, sc.detach().reshape(n_param, c), sh.detach().reshape(n_param, c), eps,
+                                     nb, affine, round_s=False)
+    torch.testing.assert_close(so, st.detach(), rtol=1e-13, atol=1e-13)
+    torch.testing.assert_close(yo, yt.detach(), rtol=1e-11, atol=1e-11)
+    ds, dres, dscale, dshift, dgate = O.residual_norm_backward(dy, ds_in, st, r, g, sc.detach().reshape(n_param, c),
+                                                               eps, nb, affine)
+    torch.testing.assert_close(ds, x.grad, rtol=1e-10, atol=1e-11)
+    torch.testing.assert_close(dres, r.grad, rtol=1e-10, atol=1e-11)
+    if affine:       # per-batch partial gradients add up to the gradient of the shared parameter
+        dscale, dshift = dscale.sum(0), dshift.sum(0)
+    torch.testing.assert_close(dscale.reshape(sc.shape), sc.grad, rtol=1e-10, atol=1e-11)
+    torch.testing.assert_close(dshift.reshape(sh.shape), sh.grad, rtol=1e-10, atol=1e-11)
+    if gated:
+        torch.testing.assert_close(dgate.reshape(g.shape), g.grad, rtol=1e-10, atol=1e-11)
+    else:
+        assert dgate is None and dres is ds
+    # with rounding, s is exactly the bf16 rounding of the unrounded sum, and ds_in = None drops that term
+    sr, _ = O.residual_norm_forward(x, r, g, sc.detach().reshape(n_param, c), sh.detach().reshape(n_param, c), eps, nb, affine)
+    torch.testing.assert_close(sr, st.detach().bfloat16().double(), rtol=0, atol=0)
+    ds0 = O.residual_norm_backward(dy, None, st, r, g, sc.detach().reshape(n_param, c), eps, nb, affine)[0]
+    torch.testing.assert_close(ds0 + ds_in, ds, rtol=1e-12, atol=1e-12)
+
+
 def test_chunked_param_grads_match_unchunked():
     nb, s, c, eps = 2, 37, 24, 1e-6
     x, sc, dy = rnd(nb, s, c, seed=27).bfloat16(), rnd(nb, c, seed=28, scale=0.1), rnd(nb, s, c, seed=29).bfloat16()
