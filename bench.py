@@ -66,7 +66,9 @@ class GpuWorkload:
         dev = torch.device("cuda:0")
         self.rows, self.cols = w.rows, w.cols
         self.ref = w.contract == "reference"
-        self.nb = w.param_shape[0] if w.op in ("adaln", "gate") and not self.ref else 1
+        self.res = w.op in ("resnorm", "resnorm_gated")
+        self.gated = w.op == "resnorm_gated"
+        self.nb = w.param_shape[0] if (w.op in ("adaln", "gate") or self.res) and not self.ref else 1
         self.rpb = self.rows // self.nb
         g = torch.Generator(device=dev).manual_seed(seed)
         bf = torch.bfloat16
@@ -79,12 +81,22 @@ class GpuWorkload:
             s = {"x": randn(self.rows, self.cols), "dy": randn(self.rows, self.cols),
                  "y": torch.empty(self.rows, self.cols, dtype=bf, device=dev),
                  "dx": torch.empty(self.rows, self.cols, dtype=bf, device=dev)}
+            if self.res:
+                s["r"], s["ds_in"] = randn(self.rows, self.cols), randn(self.rows, self.cols)
+                s["s"] = torch.empty(self.rows, self.cols, dtype=bf, device=dev)
+                s["dr"] = torch.empty(self.rows, self.cols, dtype=bf, device=dev) if self.gated else None
             if self.ref:
                 s["rstd"] = torch.empty(self.rows, dtype=torch.float32, device=dev)
                 if w.op == "adaln":
                     s["x_norm"] = torch.empty(self.rows, self.cols, dtype=bf, device=dev)
             self.sets.append(s)
-        if w.op == "rope":
+        if self.res:
+            self.p0 = randn(self.nb, self.cols, scale=0.1, offset=1.0 if self.gated else 0.0)   # scale / weight
+            self.p1 = randn(self.nb, self.cols, scale=0.1)                                      # shift / bias
+            self.gate = randn(self.nb, self.cols, scale=0.5) if self.gated else None
+            self.n_acc = 3 if self.gated else 2
+            ws_bytes = self.lib.tt_residual_norm_backward_workspace_bytes(self.rows, self.cols, self.rpb, int(self.gated))
+        elif w.op == "rope":
             self.p0 = randn(self.cols, scale=0.1, offset=1.0)              # gamma
             ang = 3.0 * torch.randn(w.shape[-2], w.head_dim // 2, generator=g, device=dev, dtype=torch.float32)
             self.p1 = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()   # fp32 (cos, sin) table
@@ -110,12 +122,18 @@ class GpuWorkload:
         gdt = bf if self.ref else torch.float32
         self.g0 = torch.empty(self.nb, self.cols, dtype=gdt, device=dev)
         self.g1 = torch.empty(self.nb, self.cols, dtype=gdt, device=dev)
+        self.g2 = torch.empty(self.nb, self.cols, dtype=gdt, device=dev)
         self.n_partials = ctypes.c_int(0)
         self.stream = torch.cuda.current_stream().cuda_stream
 
     def fwd(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.ref and self.w.op == "adaln":
+        ptr = lambda t: None if t is None else t.data_ptr()
+        if self.res:
+            self.cabi.call("tt_residual_norm_forward", s["s"].data_ptr(), s["y"].data_ptr(), s["x"].data_ptr(),
+                           s["r"].data_ptr(), ptr(self.gate), self.nb, self.p0.data_ptr(), self.p1.data_ptr(), self.nb,
+                           int(self.gated), None, None, self.rows, self.cols, self.rpb, self.w.eps, self.stream)
+        elif self.ref and self.w.op == "adaln":
             self.cabi.call("tt_launch_adaln_forward", s["y"].data_ptr(), s["x_norm"].data_ptr(), s["x"].data_ptr(),
                            self.p0.data_ptr(), self.p1.data_ptr(), self.rows, self.cols, self.w.eps,
                            s["rstd"].data_ptr(), self.stream)
@@ -138,7 +156,14 @@ class GpuWorkload:
 
     def bwd_partials(self, i):
         s = self.sets[i % len(self.sets)]
-        if self.ref and self.w.op == "adaln":   # one entry point: streaming kernel + reduction of its partials
+        ptr = lambda t: None if t is None else t.data_ptr()
+        if self.res:                            # one entry point: streaming kernel + reduction of its partials
+            self.cabi.call("tt_residual_norm_backward", s["dx"].data_ptr(), ptr(s["dr"]), self.g0.data_ptr(),
+                           self.g1.data_ptr(), self.g2.data_ptr() if self.gated else None, s["dy"].data_ptr(),
+                           s["ds_in"].data_ptr(), s["s"].data_ptr(), s["r"].data_ptr() if self.gated else None,
+                           ptr(self.gate), self.nb, self.p0.data_ptr(), self.nb, int(self.gated),
+                           self.ws.data_ptr(), self.ws.numel(), self.rows, self.cols, self.rpb, self.w.eps, self.stream)
+        elif self.ref and self.w.op == "adaln":   # one entry point: streaming kernel + reduction of its partials
             self.cabi.call("tt_launch_adaln_backward", s["dx"].data_ptr(), self.g0.data_ptr(), self.g1.data_ptr(),
                            s["dy"].data_ptr(), s["x_norm"].data_ptr(), self.p0.data_ptr(), s["rstd"].data_ptr(),
                            self.rows, self.cols, self.ws.data_ptr(), self.ws.numel(), self.stream)
@@ -165,7 +190,7 @@ class GpuWorkload:
                            self.rows, self.cols, self.w.eps, self.stream)
 
     def reduce(self):
-        if self.w.op in ("gate", "rope") or self.ref:
+        if self.w.op in ("gate", "rope") or self.ref or self.res:
             return
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
@@ -235,7 +260,10 @@ def cpu_baseline(w, seconds):
     sample_rows = min(w.shape[1], 16384)
     t = make_inputs(w, seed=0, rows=sample_rows)
     elements = t["x"].numel()
-    if w.op == "rope":
+    if w.op in ("resnorm", "resnorm_gated"):
+        fn = lambda: E.eager_residual_norm_fwd_bwd(t["x"], t["residual"], t.get("gate"), t["scale"], t["shift"], t["dy"],
+                                                   t["ds_in"], w.eps, w.op == "resnorm_gated")
+    elif w.op == "rope":
         fn = lambda: E.eager_rmsnorm_rope_fwd_bwd(t["x"], t["gamma"], t["freqs"], t["dy"], w.eps, w.head_dim)
     elif w.op == "gate":
         fn = lambda: E.eager_gate_fwd_bwd(t["x"], t["gate"], t["residual"], t["dy"])

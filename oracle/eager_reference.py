@@ -71,6 +71,24 @@ def eager_gate_fwd_bwd(x, gate, residual, dy):
     return out.detach(), xr.grad, gr.grad, rr.grad
 
 
+def eager_residual_norm_fwd_bwd(x, residual, gate, scale, shift, dy, ds_in, eps, affine):
+    """The unfused sequence of teletron/models/wan/wan_model.py:239-241 in eager bf16: the residual
+    update (GateModule, or a plain add), then nn.LayerNorm (``affine``: weight = scale, bias = shift)
+    or LayerNorm without affine + modulate; gradients arrive at both outputs.
+    Returns (s, y, dx, dresidual)."""
+    c = x.shape[-1]
+    leaves = [t.detach().clone().requires_grad_(True) for t in (x, residual, scale, shift)]
+    xr, rr, sc, sh = leaves
+    gr = gate.detach().clone().requires_grad_(True) if gate is not None else None
+    s = xr + (gr * rr if gr is not None else rr)
+    if affine:
+        y = torch.nn.functional.layer_norm(s, (c,), sc.reshape(-1), sh.reshape(-1), eps)
+    else:
+        y = torch.nn.functional.layer_norm(s, (c,), None, None, eps) * (1 + sc) + sh
+    torch.autograd.backward([y, s], [dy, ds_in])
+    return s.detach(), y.detach(), xr.grad, rr.grad
+
+
 def eager_rope_apply(x, freqs, num_heads):
     """rope_apply of teletron/models/wan/wan_model.py:105-110: float64 complex multiply per head.
     ``freqs`` is complex [S, 1, head_dim/2]."""

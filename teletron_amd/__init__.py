@@ -4,11 +4,12 @@ The compute path is hand-written HIP for gfx950 in ``libteletron_op.so`` (C ABI,
 ``include/teletron_op.h``); Python only validates, allocates and launches.
 """
 from .functional import (AdaLNModelFunction, FusedAdaLN, FusedGate, FusedRMSNorm, GateResidualFunction,
-                         RMSNormModelFunction, RMSNormRopeFunction, adaln_modulate, rms_norm)
+                         RMSNormModelFunction, RMSNormRopeFunction, ResidualNormFunction, adaln_modulate,
+                         residual_adaln, residual_layer_norm, rms_norm)
 from . import cabi, ops, swap_in, workloads
 
 __all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "GateResidualFunction", "RMSNormRopeFunction", "FusedAdaLN", "FusedRMSNorm", "FusedGate",
-           "adaln_modulate", "rms_norm", "cabi", "ops", "swap_in", "workloads", "install_reference_modules"]
+           "ResidualNormFunction", "residual_adaln", "residual_layer_norm", "adaln_modulate", "rms_norm", "cabi", "ops", "swap_in", "workloads", "install_reference_modules"]
 
 
 def install_reference_modules() -> None:

@@ -211,20 +211,22 @@ KernelInfo lookup_gate(bool narrow, int idx, bool full) {
 
 // Residual update fused with the following LayerNorm (wide rows only): forward streams two
 // inputs, backward three (four with a gate).
+// Measured at 75600 x 5120: with two to four streamed inputs and one or two outputs about five
+// waves per workgroup stream best (forward 519 us with 5 waves, 533 with 10; gated backward 786 us
+// with 5 waves against 2437 with 10, which also spills).
+constexpr int res_waves_Q(int W) { return W >= 4 ? 1 : (5 + W / 2) / W; }
 constexpr int res_fwd_Q(int W, int P) {
 #ifdef TT_RES_FWD_Q
   return TT_RES_FWD_Q * W > 16 ? 1 : TT_RES_FWD_Q;
 #else
-  return bwd_wide_Q(W, P);
+  return res_waves_Q(W);
 #endif
 }
 constexpr int res_bwd_Q(int W, int P, bool gated) {
 #ifdef TT_RES_BWD_Q
   return TT_RES_BWD_Q * W > 16 ? 1 : TT_RES_BWD_Q;
 #else
-  int q = bwd_wide_Q(W, P);
-  while (q > 1 && W * q > 8) --q;   // three or four streamed inputs: at most 8 waves, 256 VGPRs per lane
-  return q;
+  return res_waves_Q(W);
 #endif
 }
 template <int W, int P, bool FULL, bool GATED>

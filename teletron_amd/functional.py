@@ -130,6 +130,71 @@ class GateResidualFunction(Function):
                 dres if ctx.needs_input_grad[2] else None)
 
 
+class ResidualNormFunction(Function):
+    """``apply(x, residual, gate, scale, shift, epsilon, affine) -> (s, y)``: the residual update of
+    a DiT block and the normalisation that reads it, one kernel each way
+    (``teletron/models/wan/wan_model.py:239-241``).  ``s = x + gate * residual`` (``gate`` None:
+    ``x + residual``); ``y = LayerNorm(s) * (1 + scale) + shift``, or ``LayerNorm(s) * scale + shift``
+    with ``affine`` (scale / shift = weight / bias of ``nn.LayerNorm``).  Backward adds the gradients
+    arriving at ``s`` and at ``y`` in fp32 and rounds once."""
+
+    @staticmethod
+    def forward(ctx, x, residual, gate, scale, shift, epsilon, affine):
+        ctx.eps, ctx.affine = float(epsilon), bool(affine)
+        ctx.set_materialize_grads(False)
+        ctx.metas = [None if t is None else (t.shape, t.dtype) for t in (gate, scale, shift)]
+        bf = torch.bfloat16
+        gate_c = None if gate is None else gate.detach().to(bf).contiguous()
+        scale_c = scale.detach().to(bf).contiguous()
+        residual = residual.contiguous()
+        s, y = ops.residual_norm_forward(x.contiguous(), residual, gate_c, scale_c, shift.detach(), ctx.eps, ctx.affine)
+        ctx.save_for_backward(s, residual if gate is not None else None, gate_c, scale_c)
+        return s, y
+
+    @staticmethod
+    def backward(ctx, grad_s, grad_y):
+        s, residual, gate_c, scale_c = ctx.saved_tensors
+        if grad_y is None:
+            grad_y = torch.zeros_like(s)
+        dx, dr, dscale, dshift, dgate = ops.residual_norm_backward(
+            grad_y.contiguous(), None if grad_s is None else grad_s.contiguous(), s, residual, gate_c, scale_c,
+            ctx.eps, ctx.affine)
+
+        def param_grad(g, meta, needed):
+            if not needed or g is None:
+                return None
+            shape, dtype = meta
+            n = 1
+            for d in shape:
+                n *= d
+            if g.numel() != n:            # one parameter vector shared by several batches
+                g = g.sum(dim=0)
+            return g.to(dtype).reshape(shape)
+
+        need = ctx.needs_input_grad
+        return (dx if need[0] else None, dr if need[1] else None, param_grad(dgate, ctx.metas[0], need[2]),
+                param_grad(dscale, ctx.metas[1], need[3]), param_grad(dshift, ctx.metas[2], need[4]), None, None)
+
+
+def residual_adaln(x, residual, gate, shift, scale, eps: float = 1e-6):
+    """``s = x + gate * residual`` (gate None: ``x + residual``) and
+    ``modulate(layer_norm(s), shift, scale)``; returns ``(s, y)``.  Argument order of ``modulate``.
+    Shapes without a fused kernel (rows of at most 256 elements) run the two fused halves."""
+    if ops.residual_norm_supported(x):
+        return ResidualNormFunction.apply(x, residual, gate, scale, shift, eps, False)
+    s = GateResidualFunction.apply(x, gate, residual) if gate is not None else x + residual
+    return s, adaln_modulate(s, shift, scale, eps)
+
+
+def residual_layer_norm(x, residual, gate, weight, bias, eps: float = 1e-5):
+    """``s = x + gate * residual`` (gate None: ``x + residual``) and
+    ``F.layer_norm(s, weight, bias)``; returns ``(s, y)``."""
+    if ops.residual_norm_supported(x):
+        return ResidualNormFunction.apply(x, residual, gate, weight, bias, eps, True)
+    s = GateResidualFunction.apply(x, gate, residual) if gate is not None else x + residual
+    return s, torch.nn.functional.layer_norm(s, (s.shape[-1],), weight, bias, eps)
+
+
 class FusedGate(nn.Module):
     """Drop-in for ``GateModule`` (``teletron/models/wan/wan_model.py:205-210``): ``forward(x, gate, residual)``."""
 

@@ -23,6 +23,12 @@ ships no code that performs the swap.  This module does it by patching *instance
       ``__mul__`` / ``__add__`` do the same.
   Anything else done to a token raises, so a missed consumer cannot silently compute garbage.
 
+* with ``blocks=True`` every ``DiTBlock`` (``wan_model.py:231-244``) additionally gets a ``forward``
+  that fuses each residual update with the normalisation reading its result: the gated
+  self-attention update with the affine ``norm3``, and the cross-attention update with
+  ``norm2`` + modulate (:func:`fused_dit_block_forward`); 24 instead of 30 bytes per element move
+  through HBM for the block's residual/normalisation work in forward, 40 instead of 60 in backward.
+
 Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` all-reduces dscale/dshift over the
 context-parallel group (``core/context_parallel/layers.py:49-52``); with a group of size 1 that is
 the identity, which is what the fused op returns.
@@ -36,7 +42,8 @@ from typing import Callable, Iterable, Optional
 import torch
 import torch.nn as nn
 
-from .functional import AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction
+from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, adaln_modulate,
+                         residual_adaln, residual_layer_norm)
 
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
@@ -139,12 +146,43 @@ def _is_plain_layernorm(m) -> bool:
     return (isinstance(m, nn.LayerNorm) and not m.elementwise_affine and len(m.normalized_shape) == 1)
 
 
+BLOCK_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock")   # wan_model.py:212-244, parallel_wan_model.py:12-37
+
+
+def fused_dit_block_forward(self, x, context, t_mod, freqs):
+    """``DiTBlock.forward`` (``wan_model.py:231-244``; ``parallel_wan_model.py:18-37`` is the same
+    sequence) with the norm + modulate pairs and both residual updates on the fused kernels.  The
+    sub-modules (``self_attn``, ``cross_attn``, ``ffn``) and all parameters are used as they are."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16):
+        return type(self).forward(self, x, context, t_mod, freqs)
+    shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+        self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
+    input_x = adaln_modulate(x, shift_msa, scale_msa, self.norm1.eps)
+    attn_output = self.self_attn(input_x, freqs)
+    # x = gate(x, gate_msa, attn_output); norm3(x)
+    x, normed = residual_layer_norm(x, attn_output, gate_msa, self.norm3.weight, self.norm3.bias, self.norm3.eps)
+    # x = x + cross_attn(norm3(x), context); modulate(norm2(x), shift_mlp, scale_mlp)
+    x, input_x = residual_adaln(x, self.cross_attn(normed, context), None, shift_mlp, scale_mlp, self.norm2.eps)
+    return GateResidualFunction.apply(x, gate_mlp, self.ffn(input_x))
+
+
+def _is_dit_block(m: nn.Module) -> bool:
+    if type(m).__name__ not in BLOCK_CLASSES:
+        return False
+    if type(m).__name__ != "DiTBlock" and torch.distributed.is_available() and torch.distributed.is_initialized() \
+            and torch.distributed.get_world_size() > 1:
+        return False      # the context-parallel block all-reduces its modulation gradients over the group
+    return (all(hasattr(m, a) for a in ("modulation", "self_attn", "cross_attn", "ffn", "norm1", "norm2"))
+            and isinstance(getattr(m, "norm3", None), nn.LayerNorm) and m.norm3.elementwise_affine)
+
+
 def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool = True, adaln: bool = True,
-            gate: bool = True) -> dict:
+            gate: bool = True, blocks: bool = False) -> dict:
     """Patch ``model`` in place.  ``namespaces`` are Python modules (e.g. the imported
     ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
-    tokens.  Returns counts of what was swapped."""
-    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0}
+    tokens.  ``blocks`` also replaces the forward of whole DiT blocks (see the module docstring).
+    Returns counts of what was swapped."""
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0}
     for ns in namespaces:
         fn = getattr(ns, "modulate", None)
         if callable(fn) and not hasattr(fn, "__wrapped__"):
@@ -157,6 +195,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__:
             module.forward = types.MethodType(_fused_gate_forward, module)
             counts["gate"] += 1
+        if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(fused_dit_block_forward, module)
+            counts["block"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
             for attr in MODULATE_ATTRS:
                 fn = getattr(module, attr, None)

@@ -15,7 +15,7 @@ import torch
 @dataclass(frozen=True)
 class Workload:
     name: str
-    op: str                      # "adaln" | "rmsnorm" | "rope" | "gate"
+    op: str                      # "adaln" | "rmsnorm" | "rope" | "gate" | "resnorm" | "resnorm_gated"
     shape: Tuple[int, ...]       # activation shape, normalised dim last
     param_shape: Tuple[int, ...]
     eps: float = 1e-6
@@ -50,6 +50,13 @@ class Workload:
             fwd = 4 * e + n_param * 2 + table
             bwd = 6 * e + n_param * 2 + n_param * 4 + table
             return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
+        if self.op in ("resnorm", "resnorm_gated"):
+            # forward: x, r in; s, y out.  backward: s, dy, ds_in (+ r) in; dx (+ dr) out.
+            n_in = 4 if self.op == "resnorm_gated" else 3
+            n_vec = 3 if self.op == "resnorm_gated" else 2
+            fwd = 8 * e + n_vec * n_param * 2
+            bwd = 2 * (n_in + n_in - 2) * e + (n_vec - 1) * n_param * 2 + n_vec * n_param * 4
+            return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
         if self.op == "gate":        # out = x + gate * residual: two activations in, one out, each way
             fwd = 6 * e + n_param * 2
             bwd = 6 * e + n_param * 2 + n_param * 4
@@ -79,6 +86,10 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
              note="the reference's own AdaLN width, through its launcher signatures"),
     Workload("rmsnorm_hunyuan_head_reference_contract", "rmsnorm", (1, 118800, 24, 128), (128,), contract="reference",
              note="the reference's own RMSNorm width, through its launcher signatures"),
+    Workload("residual_adaln_wan14b", "resnorm", (1, 75600, 5120), (1, 1, 5120),
+             note="x + cross_attn(..) fused with norm2 + modulate"),
+    Workload("gated_residual_layernorm_wan14b", "resnorm_gated", (1, 75600, 5120), (1, 1, 5120),
+             note="gate(x, gate_msa, attn) fused with the affine norm3"),
     Workload("gate_wan14b", "gate", (1, 75600, 5120), (1, 1, 5120), note="gated residual add after each AdaLN site"),
 ]}
 
@@ -95,7 +106,16 @@ def make_inputs(w: Workload, seed: int = 0, device="cpu", rows: Optional[int] = 
     g = torch.Generator(device="cpu").manual_seed(seed)
     x = torch.randn(shape, generator=g, dtype=torch.float32)
     out = {}
-    if w.op == "gate":
+    if w.op in ("resnorm", "resnorm_gated"):
+        out["residual"] = torch.randn(shape, generator=g, dtype=torch.float32)
+        out["ds_in"] = torch.randn(shape, generator=g, dtype=torch.float32)
+        if w.op == "resnorm_gated":      # gate + affine LayerNorm (weight, bias)
+            out["gate"] = 0.5 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+            out["scale"] = 1.0 + 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        else:
+            out["scale"] = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+        out["shift"] = 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
+    elif w.op == "gate":
         out["gate"] = 0.5 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
         out["residual"] = torch.randn(shape, generator=g, dtype=torch.float32)
     elif w.op == "adaln":

@@ -143,7 +143,7 @@ def test_swap_in_matches_eager_model(monkeypatch):
     assert S.swap_in_if_requested(model, [ns]) is None
     monkeypatch.setenv("FUSED_KERNELS", "1")
     counts = S.swap_in_if_requested(model, [ns])
-    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4}, counts
+    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4, "block": 0}, counts
     assert isinstance(model.blocks[0].norm3, nn.LayerNorm)               # affine LayerNorm untouched
     assert list(model.state_dict().keys()) == keys_before                 # checkpoint compatible
     try:
@@ -157,7 +157,85 @@ def test_swap_in_matches_eager_model(monkeypatch):
         assert rel(a, b) < 2e-2
     worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
     assert worst < 2e-2, worst
-    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0}   # idempotent on the model
+    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0, "block": 0}   # idempotent on the model
+
+
+class RefAttention(nn.Module):
+    """Stand-in for SelfAttention / CrossAttention: only the call signature matters here."""
+
+    def __init__(self, dim, cross):
+        super().__init__()
+        self.proj, self.cross = nn.Linear(dim, dim), cross
+
+    def forward(self, x, other):
+        return self.proj(x) * 0.5 + (other.mean(dim=1, keepdim=True) if self.cross else 0.0)
+
+
+def make_ref_block(dim, eps=1e-6):
+    """A block with the attributes and the forward of wan_model.py:212-244."""
+
+    class DiTBlock(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.self_attn, self.cross_attn = RefAttention(dim, False), RefAttention(dim, True)
+            self.norm1 = nn.LayerNorm(dim, eps=eps, elementwise_affine=False)
+            self.norm2 = nn.LayerNorm(dim, eps=eps, elementwise_affine=False)
+            self.norm3 = nn.LayerNorm(dim, eps=eps)
+            self.ffn = nn.Sequential(nn.Linear(dim, 2 * dim), nn.GELU(approximate="tanh"), nn.Linear(2 * dim, dim))
+            self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
+            self.gate, self.gate2 = GateModule(), GateModule()
+
+        def forward(self, x, context, t_mod, freqs):
+            shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
+                self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
+            input_x = modulate(self.norm1(x), shift_msa, scale_msa)
+            attn_output = self.self_attn(input_x, freqs)
+            x = self.gate(x, gate_msa, attn_output)
+            x = x + self.cross_attn(self.norm3(x), context)
+            input_x = modulate(self.norm2(x), shift_mlp, scale_mlp)
+            x = self.gate2(x, gate_mlp, self.ffn(input_x))
+            return x
+
+    return DiTBlock()
+
+
+@pytest.mark.parametrize("dim", [512, 256])      # 256: rows too short for the fused pair, the halves run
+def test_block_level_swap_in_matches_eager_block(dim):
+    from teletron_amd import swap_in as S
+    torch.manual_seed(3)
+    bsz, seq = 2, 80
+    model = nn.ModuleList([make_ref_block(dim), make_ref_block(dim)]).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        for b in model:
+            b.norm3.weight.add_(0.2 * torch.randn_like(b.norm3.weight))
+            b.norm3.bias.add_(0.2 * torch.randn_like(b.norm3.bias))
+    g = torch.Generator().manual_seed(4)
+    mk = lambda *s, scale=1.0: (scale * torch.randn(*s, generator=g)).to(torch.bfloat16).to(DEV)
+    inputs = [mk(bsz, seq, dim), mk(bsz, 7, dim), mk(bsz, 6, dim, scale=0.2)]
+    dy = mk(bsz, seq, dim)
+
+    class Stack(nn.Module):
+        def __init__(self, blocks):
+            super().__init__()
+            self.blocks = blocks
+
+        def forward(self, x, context, t_mod):
+            for b in self.blocks:
+                x = b(x, context, t_mod, None)
+            return x
+
+    stack = Stack(model)
+    keys_before = list(stack.state_dict().keys())
+    out_e, gin_e, gp_e = run(stack, inputs, dy)
+    counts = S.swap_in(stack, blocks=True)
+    assert counts["block"] == 2 and counts["gate"] == 4 and counts["layernorm"] == 4, counts
+    assert list(stack.state_dict().keys()) == keys_before
+    out_f, gin_f, gp_f = run(stack, inputs, dy)
+    assert rel(out_f, out_e) < 5e-3
+    for a, b in zip(gin_f, gin_e):
+        assert rel(a, b) < 2e-2
+    worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
+    assert worst < 2e-2, worst
 
 
 def test_deferred_norm_refuses_other_uses():
