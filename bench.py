@@ -47,7 +47,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
     ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched,"
-                                      "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract",
+                                      "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
+                                      "residual_adaln_wan14b,gated_residual_layernorm_wan14b",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "

@@ -83,3 +83,78 @@ def test_residual_norm_reproducible_and_refuses_narrow_rows():
         ops.residual_norm_forward(xs, xs, None, xs[0], xs[0], 1e-6)
     with pytest.raises(ValueError):          # 3 gate vectors do not pair with 2 modulation vectors
         ops.residual_norm_forward(x, r, rand_bf16(3, 2048, seed=1).to(DEV), scale, shift, 1e-6)
+
+
+@pytest.mark.parametrize("name", ["residual_adaln_wan14b", "gated_residual_layernorm_wan14b"])
+def test_residual_norm_full_size(name):
+    """The benchmark shapes at full size: sampled rows against the float64 oracle, every element
+    against a plain torch fp32 evaluation on the GPU, parameter gradients against a streamed
+    float64 accumulation of that evaluation."""
+    from teletron_amd import ops
+    from teletron_amd.workloads import WORKLOADS, make_inputs
+    from test_gpu_configs import sample_rows, whole_tensor_check
+    w = WORKLOADS[name]
+    gated = affine = w.op == "resnorm_gated"
+    c, eps = w.cols, w.eps
+    t = make_inputs(w, seed=0)
+    d = {k: v.to(DEV) for k, v in t.items()}
+    gate = d.get("gate")
+    s, y = ops.residual_norm_forward(d["x"], d["residual"], gate, d["scale"], d["shift"], eps, affine)
+    dx, dr, dscale, dshift, dgate = ops.residual_norm_backward(d["dy"], d["ds_in"], s, d["residual"], gate, d["scale"], eps, affine)
+    torch.cuda.synchronize()
+
+    idx = sample_rows(w.rows, 512, seed=2)
+    rows = lambda v: v.reshape(-1, c)[idx]
+    gate_c = None if gate is None else t["gate"].reshape(1, c)
+    so, _ = O.residual_norm_forward(rows(t["x"]), rows(t["residual"]), gate_c, t["scale"], t["shift"], eps, 1, affine)
+    s_rows = s.reshape(-1, c)[idx.to(DEV)].cpu()
+    assert_bf16_close(s_rows, so, "s")
+    yo = O.adaln_forward(s_rows, O._param(t["scale"], 1, c) - (1.0 if affine else 0.0), t["shift"], eps, 1)[0]
+    assert_bf16_close(y.reshape(-1, c)[idx.to(DEV)], yo, "y")
+    dso, dro, _, _, _ = O.residual_norm_backward(rows(t["dy"]), rows(t["ds_in"]), s_rows, rows(t["residual"]), gate_c,
+                                                 t["scale"], eps, 1, affine)
+    assert_bf16_close(dx.reshape(-1, c)[idx.to(DEV)], dso, "dx")
+    if gated:
+        assert_bf16_close(dr.reshape(-1, c)[idx.to(DEV)], dro, "dresidual")
+
+    x2, r2, s2, dy2, ds2 = (v.reshape(-1, c) for v in (d["x"], d["residual"], s, d["dy"], d["ds_in"]))
+    gf = gate.float().reshape(1, c) if gated else None
+    mult = d["scale"].float().reshape(1, c) + (0.0 if affine else 1.0)
+    shf = d["shift"].float().reshape(1, c)
+
+    def ref_s(r0, r1):
+        return x2[r0:r1].float() + (gf * r2[r0:r1].float() if gated else r2[r0:r1].float())
+
+    def norm_parts(r0, r1):
+        sf = s2[r0:r1].float()
+        mean = sf.mean(-1, keepdim=True)
+        rstd = torch.rsqrt((sf - mean).pow(2).mean(-1, keepdim=True) + eps)
+        return (sf - mean) * rstd, rstd
+
+    def ref_y(r0, r1):
+        return norm_parts(r0, r1)[0] * mult + shf
+
+    def ref_ds(r0, r1):
+        xh, rstd = norm_parts(r0, r1)
+        g = dy2[r0:r1].float() * mult
+        return ds2[r0:r1].float() + rstd * (g - g.mean(-1, keepdim=True) - xh * (g * xh).mean(-1, keepdim=True))
+
+    whole_tensor_check(s, ref_s)
+    whole_tensor_check(y, ref_y)
+    whole_tensor_check(dx, ref_ds)
+    if gated:
+        whole_tensor_check(dr, lambda r0, r1: gf * ref_ds(r0, r1))
+
+    acc = torch.zeros(3, c, dtype=torch.float64, device=DEV)
+    for r0 in range(0, w.rows, 8192):
+        r1 = min(r0 + 8192, w.rows)
+        xh, _ = norm_parts(r0, r1)
+        dyf = dy2[r0:r1].double()
+        acc[0] += (dyf * xh.double()).sum(0)
+        acc[1] += dyf.sum(0)
+        if gated:
+            acc[2] += (ref_ds(r0, r1).double() * r2[r0:r1].double()).sum(0)
+    assert_grad_close(dscale, acc[0].cpu(), w.rows, "dscale")
+    assert_grad_close(dshift, acc[1].cpu(), w.rows, "dshift")
+    if gated:
+        assert_grad_close(dgate / 2, acc[2].cpu() / 2, w.rows, "dgate")
