@@ -211,22 +211,30 @@ KernelInfo lookup_gate(bool narrow, int idx, bool full) {
 
 // Residual update fused with the following LayerNorm (wide rows only): forward streams two
 // inputs, backward three (four with a gate).
-// Measured at 75600 x 5120: with two to four streamed inputs and one or two outputs about five
-// waves per workgroup stream best (forward 519 us with 5 waves, 533 with 10; gated backward 786 us
-// with 5 waves against 2437 with 10, which also spills).
-constexpr int res_waves_Q(int W) { return W >= 4 ? 1 : (5 + W / 2) / W; }
+// Row groups per workgroup for the kernels with two to four streamed inputs, from sweeps on
+// MI355X: about ten waves where a lane holds one pack per tensor; with two packs per lane as many
+// row groups as fit in eight waves, which leaves the backward kernels their 170-235 VGPRs
+// (ten waves cap them at 168 and they spill).  Measured (forward / backward / gated backward, us):
+// 1536 columns 281 / 271 / 418 with 9 waves against 302 / 287 / 459 with 3; 2048: 207 / 203 / 326
+// with 12 waves against 221 / 212 / 362 with 4; 3072 x 118800 rows: 492 / 477 / 746 with 6 waves;
+// 4096 x 90000: 502 / 478 / 763 with 8 waves against 522 / 523 / 888 with 4; 5120: 519 / 525 / 786
+// with 5 waves against 533 / 595 / 2437 with 10.
+constexpr int res_waves_Q(int W, int P) {
+  const int q = P == 1 ? (10 + W / 2) / W : 8 / W;
+  return q < 1 ? 1 : q;
+}
 constexpr int res_fwd_Q(int W, int P) {
 #ifdef TT_RES_FWD_Q
   return TT_RES_FWD_Q * W > 16 ? 1 : TT_RES_FWD_Q;
 #else
-  return res_waves_Q(W);
+  return res_waves_Q(W, P);
 #endif
 }
 constexpr int res_bwd_Q(int W, int P, bool gated) {
 #ifdef TT_RES_BWD_Q
   return TT_RES_BWD_Q * W > 16 ? 1 : TT_RES_BWD_Q;
 #else
-  return res_waves_Q(W);
+  return res_waves_Q(W, P);
 #endif
 }
 template <int W, int P, bool FULL, bool GATED>
