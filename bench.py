@@ -50,6 +50,7 @@ def parse_args():
                                       "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
                                       "residual_adaln_wan14b,gated_residual_layernorm_wan14b",
                     help="comma list of further workloads reported under 'also'")
+    ap.add_argument("--no-eager-gpu", action="store_true", help="skip timing the eager PyTorch expressions on the GPU")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
                          "that hardware byte counters collected over this run can be scaled against it")
@@ -252,6 +253,56 @@ class GpuWorkload:
                       "reduce": [e[2].elapsed_time(e[3]) * 1e3 for e in ev]}
 
 
+def eager_gpu(w, iters=5):
+    """What runs on this GPU when the fused kernels are switched off: the model code's own eager
+    PyTorch expressions (teletron/models/wan/wan_model.py:77-78,113-124,205-210,239-241) in bf16
+    with autograd, on synthetic tensors of the workload's shape.  Milliseconds per forward+backward."""
+    import torch
+    import torch.nn.functional as F
+    dev, bf, c = "cuda:0", torch.bfloat16, w.cols
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape, scale=1.0, offset=0.0: (offset + scale * torch.randn(*shape, generator=g, device=dev)).to(bf)
+    shape = tuple(w.shape)
+    nb = w.param_shape[0] if len(w.param_shape) == 3 else 1
+    pshape = (nb, 1, c) if len(shape) == 3 else (c,)
+    x, dy = rnd(*shape).requires_grad_(True), rnd(*shape)
+    if w.op == "adaln":
+        scale, shift = rnd(*pshape, scale=0.1).requires_grad_(True), rnd(*pshape, scale=0.1).requires_grad_(True)
+        fn = lambda: torch.autograd.backward([F.layer_norm(x, (c,), eps=w.eps) * (1 + scale) + shift], [dy])
+    elif w.op == "rmsnorm":
+        weight = rnd(c, scale=0.1, offset=1.0).requires_grad_(True)
+
+        def fn():
+            xf = x.float()
+            y = (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + w.eps)).to(bf) * weight
+            y.backward(dy)
+    elif w.op == "gate":
+        gate, r = rnd(*pshape, scale=0.5).requires_grad_(True), rnd(*shape).requires_grad_(True)
+        fn = lambda: (x + gate * r).backward(dy)
+    elif w.op in ("resnorm", "resnorm_gated"):
+        r, ds_in = rnd(*shape).requires_grad_(True), rnd(*shape)
+        scale, shift = rnd(*pshape, scale=0.1).requires_grad_(True), rnd(*pshape, scale=0.1).requires_grad_(True)
+        gate = rnd(*pshape, scale=0.5).requires_grad_(True) if w.op == "resnorm_gated" else None
+
+        def fn():
+            s = x + (gate * r if gate is not None else r)
+            if gate is not None:      # gate + affine LayerNorm (norm3)
+                y = F.layer_norm(s, (c,), scale.reshape(-1)[:c], shift.reshape(-1)[:c], w.eps)
+            else:                     # residual add + norm2 + modulate
+                y = F.layer_norm(s, (c,), eps=w.eps) * (1 + scale) + shift
+            torch.autograd.backward([y, s], [dy, ds_in])
+    else:
+        return None
+    for _ in range(2):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters * 1e3
+
+
 def cpu_baseline(w, seconds):
     """PyTorch-eager fwd + autograd bwd of the same op on the host CPU, bounded row sample."""
     import torch
@@ -349,6 +400,11 @@ def main():
         "forward_frac_of_copy": round(r["fwd_gbps"] / c["copy"], 4),
         "backward_frac_of_two_reads_one_write": round(r["bwd_gbps"] / c["two_reads_one_write"], 4),
         "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers"}
+    if not args.no_eager_gpu:
+        ms = eager_gpu(w)
+        if ms:
+            out["eager_gpu"] = {"ms_per_step": round(ms, 3), "speedup": round(ms / r["ms_per_step"], 2),
+                                "note": "the model code's eager PyTorch expressions with autograd, bf16, same GPU"}
     also = {}
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         wa = WORKLOADS[name]
@@ -356,6 +412,11 @@ def main():
         also[name] = {"value": round(ra["gbps"], 1), "unit": "GB/s", "pct_of_peak": round(100 * ra["gbps"] / HBM_PEAK_GBPS, 2),
                       "ms_per_step": round(ra["ms_per_step"], 4), "forward_us": round(ra["fwd_us"], 2),
                       "backward_streaming_us": round(ra["bwd_us"], 2), "reduce_partials_us": round(ra["reduce_us"], 2)}
+        if not args.no_eager_gpu:
+            ms = eager_gpu(wa, iters=3)
+            if ms:
+                also[name]["eager_gpu_ms_per_step"] = round(ms, 3)
+                also[name]["speedup_vs_eager_gpu"] = round(ms / ra["ms_per_step"], 2)
     if also:
         out["also"] = also
     if args.calibrate_copy:
