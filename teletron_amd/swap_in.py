@@ -29,9 +29,11 @@ ships no code that performs the swap.  This module does it by patching *instance
   ``norm2`` + modulate (:func:`fused_dit_block_forward`); 24 instead of 30 bytes per element move
   through HBM for the block's residual/normalisation work in forward, 40 instead of 60 in backward.
 
-Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` all-reduces dscale/dshift over the
-context-parallel group (``core/context_parallel/layers.py:49-52``); with a group of size 1 that is
-the identity, which is what the fused op returns.
+Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` / ``gate_with_cp_grad_reduce``
+all-reduce their parameter gradients over the context-parallel group
+(``core/context_parallel/layers.py:31-36,46-53``); with a group of size 1 that is the identity,
+which is what the fused ops return.  While ``torch.distributed`` runs with more than one rank
+these callables (and the context-parallel block's forward) are therefore left as they are.
 """
 from __future__ import annotations
 
@@ -48,6 +50,8 @@ from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelF
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
 MODULATE_ATTRS = ("modulate", "modulate_with_cp_grad_reduce")
+GATE_ATTRS = ("gate_with_cp_grad_reduce",)                   # context_parallel/layers.py:20-21, parallel_wan_model.py:26,35
+CP_ATTRS = ("modulate_with_cp_grad_reduce", "gate_with_cp_grad_reduce")
 GATE_CLASSES = ("GateModule", "ContextParallelGateModule")   # wan_model.py:205-210, context_parallel/layers.py:12-17
 
 
@@ -106,6 +110,30 @@ def fused_modulate(original: Callable) -> Callable:
 
     modulate.__wrapped__ = original
     return modulate
+
+
+def fused_gate(original: Callable) -> Callable:
+    """Wrap a ``gate(x, gate, residual)`` callable: bf16 GPU tensors take the fused kernel."""
+
+    def gate(x, gate, residual):
+        if (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16
+                and residual.dtype == torch.bfloat16 and x.shape == residual.shape):
+            return GateResidualFunction.apply(x, gate, residual)
+        return original(x, gate, residual)
+
+    gate.__wrapped__ = original
+    return gate
+
+
+def _is_cp_callable(attr: str, fn) -> bool:
+    """A context-parallel gradient-reducing callable, under its own name or assigned to another
+    attribute (``norm1.modulate = self.modulate_with_cp_grad_reduce``, hunyuan/parallel_model.py:239-244)."""
+    return attr in CP_ATTRS or getattr(fn, "__name__", "") in CP_ATTRS
+
+
+def _several_ranks() -> bool:
+    return (torch.distributed.is_available() and torch.distributed.is_initialized()
+            and torch.distributed.get_world_size() > 1)
 
 
 class DeferredLayerNorm(nn.Module):
@@ -169,8 +197,7 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
 def _is_dit_block(m: nn.Module) -> bool:
     if type(m).__name__ not in BLOCK_CLASSES:
         return False
-    if type(m).__name__ != "DiTBlock" and torch.distributed.is_available() and torch.distributed.is_initialized() \
-            and torch.distributed.get_world_size() > 1:
+    if type(m).__name__ != "DiTBlock" and _several_ranks():
         return False      # the context-parallel block all-reduces its modulation gradients over the group
     return (all(hasattr(m, a) for a in ("modulation", "self_attn", "cross_attn", "ffn", "norm1", "norm2"))
             and isinstance(getattr(m, "norm3", None), nn.LayerNorm) and m.norm3.elementwise_affine)
@@ -192,16 +219,28 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if rmsnorm and _is_rmsnorm(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(_fused_rmsnorm_forward, module)
             counts["rmsnorm"] += 1
-        if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__:
+        if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__ \
+                and not (type(module).__name__ == "ContextParallelGateModule" and _several_ranks()):
             module.forward = types.MethodType(_fused_gate_forward, module)
             counts["gate"] += 1
         if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_dit_block_forward, module)
             counts["block"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
-            for attr in MODULATE_ATTRS:
-                fn = getattr(module, attr, None)
-                if callable(fn) and not hasattr(fn, "__wrapped__"):
+            # The *_with_cp_grad_reduce callables all-reduce their parameter gradients over the
+            # context-parallel group; they are only replaced where that is the identity.  An owner
+            # whose modulation goes through one of them then keeps its LayerNorms as well.
+            attrs = [(a, getattr(module, a, None)) for a in MODULATE_ATTRS + (GATE_ATTRS if gate else ())]
+            attrs = [(a, fn) for a, fn in attrs if callable(fn) and not isinstance(fn, nn.Module)]
+            if _several_ranks() and any(_is_cp_callable(a, fn) for a, fn in attrs):
+                continue
+            for attr, fn in attrs:
+                if hasattr(fn, "__wrapped__"):
+                    continue
+                if attr in GATE_ATTRS:
+                    setattr(module, attr, fused_gate(fn))
+                    counts["gate"] += 1
+                else:
                     setattr(module, attr, fused_modulate(fn))
                     counts["modulate"] += 1
             for attr in ADALN_NORM_ATTRS:

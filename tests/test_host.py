@@ -121,3 +121,40 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     p = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert p.returncode != 0 and "one GPU" in p.stderr
+
+
+def test_swap_in_leaves_context_parallel_callables_alone_with_several_ranks(monkeypatch):
+    """The *_with_cp_grad_reduce callables all-reduce their parameter gradients over the
+    context-parallel group (teletron/core/context_parallel/layers.py:31-36,46-53); the fused
+    single-GPU ops may replace them only where that reduction is the identity."""
+    import torch.nn as nn
+    from teletron_amd import swap_in as S
+
+    def make():
+        class ContextParallelWanDitBlock(nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.norm1 = nn.LayerNorm(64, eps=1e-6, elementwise_affine=False)
+                self.norm2 = nn.LayerNorm(64, eps=1e-6, elementwise_affine=False)
+                self.norm3 = nn.LayerNorm(64, eps=1e-6)
+                self.self_attn = self.cross_attn = self.ffn = nn.Identity()
+                self.modulation = nn.Parameter(torch.zeros(1, 6, 64))
+                self.modulate_with_cp_grad_reduce = lambda x, shift, scale: x * (1 + scale) + shift
+                self.gate_with_cp_grad_reduce = lambda x, gate, residual: x + gate * residual
+        return ContextParallelWanDitBlock()
+
+    one = make()
+    counts = S.swap_in(one, blocks=True)
+    assert counts["modulate"] == 1 and counts["gate"] == 1 and counts["block"] == 1 and counts["layernorm"] == 2
+    assert hasattr(one.modulate_with_cp_grad_reduce, "__wrapped__") and hasattr(one.gate_with_cp_grad_reduce, "__wrapped__")
+    # CPU tensors fall through to the original callables and to the original forward
+    x = torch.randn(2, 3, 64)
+    assert torch.equal(one.gate_with_cp_grad_reduce(x, torch.ones(2, 1, 64), x), 2 * x)
+
+    monkeypatch.setattr(S, "_several_ranks", lambda: True)
+    many = make()
+    counts = S.swap_in(many, blocks=True)
+    assert counts["modulate"] == 0 and counts["gate"] == 0 and counts["block"] == 0 and counts["layernorm"] == 0
+    assert isinstance(many.norm1, nn.LayerNorm)
+    assert not hasattr(many.modulate_with_cp_grad_reduce, "__wrapped__")
+    assert "forward" not in many.__dict__
