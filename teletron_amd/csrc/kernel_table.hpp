@@ -57,6 +57,20 @@ constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
 
 constexpr int fwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_FWD_R; }
 constexpr int bwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_BWD_R; }
+// AdaLN backward has two barrier-coupled reductions per row; on the variants below two rows per
+// row group and tile (both rows share each exchange) hide that latency better.  Measured,
+// us at R = 1 -> R = 2: 32760 x 1536: 53.8 -> 51.9; 4 x 32760 x 1536: 200.8 -> 198.0;
+// 150000 x 2048: 300.9 -> 290.0; 118800 x 3072: 358.4 -> 348.9; 60000 x 6144: 381.2 -> 355.4;
+// 300000 x 1024: 290.7 -> 288.5.  Worse with R = 2: 512 columns (156.9 -> 169.0), 4096
+// (356.6 -> 368.8), 8192 (358.0 -> 399.5), and 5120 (ten waves: spills).  RMSNorm (one reduction
+// per row) is 2-3 % slower with R = 2 everywhere.
+constexpr int adaln_bwd_wide_R(int W, int P) {
+#ifdef TT_ADALN_BWD_R
+  return P >= 4 ? 1 : TT_ADALN_BWD_R;
+#else
+  return ((P == 1 && W >= 2 && W <= 4) || (P == 2 && (W == 3 || W == 6))) ? 2 : bwd_wide_R(W, P);
+#endif
+}
 constexpr int fwd_wide_Q(int W, int P) {
 #ifdef TT_FWD_Q
   return TT_FWD_Q * W > 16 ? 1 : TT_FWD_Q;
@@ -99,7 +113,7 @@ KernelInfo info_fwd_wide() {
 }
 template <int KIND, int W, int P, bool FULL>
 KernelInfo info_bwd_wide() {
-  constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
+  constexpr int R = KIND == kAdaLN ? adaln_bwd_wide_R(W, P) : bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
   return {reinterpret_cast<const void*>(&norm_bwd_wide<KIND, W, P, R, Q, FULL>), 64 * W * Q, Q * R, P * R};
 }
 template <int KIND, int W, int P, bool FULL>
