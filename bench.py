@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
     ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched,"
                                       "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
-                                      "residual_adaln_wan14b,gated_residual_layernorm_wan14b",
+                                      "residual_adaln_wan14b,gated_residual_layernorm_wan14b,rmsnorm_rope_hunyuan_head",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--no-eager-gpu", action="store_true", help="skip timing the eager PyTorch expressions on the GPU")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -98,9 +98,10 @@ class GpuWorkload:
             self.gate = randn(self.nb, self.cols, scale=0.5) if self.gated else None
             self.n_acc = 3 if self.gated else 2
             ws_bytes = self.lib.tt_residual_norm_backward_workspace_bytes(self.rows, self.cols, self.rpb, int(self.gated))
-        elif w.op == "rope":
+        elif w.op in ("rope", "rope_heads"):
             self.p0 = randn(self.cols, scale=0.1, offset=1.0)              # gamma
-            ang = 3.0 * torch.randn(w.shape[-2], w.head_dim // 2, generator=g, device=dev, dtype=torch.float32)
+            self.seq = w.shape[-2] if w.op == "rope" else w.shape[-3]
+            ang = 3.0 * torch.randn(self.seq, w.head_dim // 2, generator=g, device=dev, dtype=torch.float32)
             self.p1 = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()   # fp32 (cos, sin) table
             self.n_acc = 1
             ws_bytes = self.lib.tt_rmsnorm_backward_workspace_bytes(self.rows, self.cols)
@@ -142,6 +143,10 @@ class GpuWorkload:
         elif self.ref:
             self.cabi.call("tt_launch_rms_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
                            self.rows, self.cols, self.w.eps, s["rstd"].data_ptr(), self.stream)
+        elif self.w.op == "rope_heads":
+            self.cabi.call("tt_rmsnorm_rope_heads_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
+                           self.p1.data_ptr(), None, self.rows, self.cols, self.w.shape[-2], self.seq,
+                           self.w.eps, self.stream)
         elif self.w.op == "rope":
             self.cabi.call("tt_rmsnorm_rope_forward", s["y"].data_ptr(), s["x"].data_ptr(), self.p0.data_ptr(),
                            self.p1.data_ptr(), None, self.rows, self.cols, self.w.head_dim, self.w.shape[-2],
@@ -173,6 +178,10 @@ class GpuWorkload:
             self.cabi.call("tt_launch_rms_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
                            s["y"].data_ptr(), self.p0.data_ptr(), s["rstd"].data_ptr(), self.rows, self.cols,
                            self.ws.data_ptr(), self.ws.numel(), self.stream)
+        elif self.w.op == "rope_heads":    # one entry point: streaming kernel + reduction of its partials
+            self.cabi.call("tt_rmsnorm_rope_heads_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
+                           s["x"].data_ptr(), self.p0.data_ptr(), self.p1.data_ptr(), self.ws.data_ptr(),
+                           self.ws.numel(), self.rows, self.cols, self.w.shape[-2], self.seq, self.w.eps, self.stream)
         elif self.w.op == "rope":          # one entry point: streaming kernel + reduction of its partials
             self.cabi.call("tt_rmsnorm_rope_backward", s["dx"].data_ptr(), self.g0.data_ptr(), s["dy"].data_ptr(),
                            s["x"].data_ptr(), self.p0.data_ptr(), self.p1.data_ptr(), self.ws.data_ptr(),
@@ -192,7 +201,7 @@ class GpuWorkload:
                            self.rows, self.cols, self.w.eps, self.stream)
 
     def reduce(self):
-        if self.w.op in ("gate", "rope") or self.ref or self.res:
+        if self.w.op in ("gate", "rope", "rope_heads") or self.ref or self.res:
             return
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
@@ -317,6 +326,8 @@ def cpu_baseline(w, seconds):
                                                    t["ds_in"], w.eps, w.op == "resnorm_gated")
     elif w.op == "rope":
         fn = lambda: E.eager_rmsnorm_rope_fwd_bwd(t["x"], t["gamma"], t["freqs"], t["dy"], w.eps, w.head_dim)
+    elif w.op == "rope_heads":
+        fn = lambda: E.eager_rmsnorm_rope_heads_fwd_bwd(t["x"], t["gamma"], t["freqs"], t["dy"], w.eps)
     elif w.op == "gate":
         fn = lambda: E.eager_gate_fwd_bwd(t["x"], t["gate"], t["residual"], t["dy"])
     elif w.op == "adaln":

@@ -160,6 +160,23 @@ TT_API int tt_rmsnorm_rope_backward(void* dx, float* dweight, const void* dy, co
                                     int64_t rows, int64_t cols, int64_t head_dim, int64_t seq_len,
                                     float eps, void* stream);
 
+/* Per-head variant: HunyuanVideo normalises every head on its own (head_dim = 128, one weight
+ * vector shared by the heads) and applies the rotary embedding right after
+ * (teletron/models/hunyuan/model.py:92-125).  x is [rows, head_dim] in memory order
+ * [batch, token, head, head_dim], i.e. `heads` consecutive rows belong to one token; row r uses
+ * position (r / heads) % seq_len.  freqs as above: (cos, sin) per position and pair
+ * (diffusers' real cos / sin tables [seq_len, head_dim] hold each value twice: take every second
+ * column).  Tokens that take no rotation (the text tokens appended in the single-stream blocks,
+ * model.py:101-121) get (1, 0) entries.  head_dim % 8 == 0, head_dim <= 256, rows % heads == 0.
+ * Workspace: tt_rmsnorm_backward_workspace_bytes(rows, head_dim). */
+TT_API int tt_rmsnorm_rope_heads_forward(void* y, const void* x, const void* weight, const float* freqs, float* rstd,
+                                         int64_t rows, int64_t head_dim, int64_t heads, int64_t seq_len,
+                                         float eps, void* stream);
+TT_API int tt_rmsnorm_rope_heads_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
+                                          const float* freqs, void* workspace, size_t workspace_bytes,
+                                          int64_t rows, int64_t head_dim, int64_t heads, int64_t seq_len,
+                                          float eps, void* stream);
+
 /* ------------------------------------------------------------------ gated residual add
  * out = x + gate * residual, the op that follows each fused AdaLN site in a DiT block;
  * gate is [n_batches, cols] bf16, broadcast over the rows of its batch.  teletron_op has no

@@ -107,3 +107,21 @@ def eager_rmsnorm_rope_fwd_bwd(x, gamma, freqs_cs, dy, eps, head_dim):
     y = eager_rope_apply(mod(xr), freqs, x.shape[-1] // head_dim)
     y.backward(dy)
     return y.detach(), xr.grad, mod.weight.grad
+
+
+def eager_rmsnorm_rope_heads_fwd_bwd(x, gamma, freqs_cs, dy, eps):
+    """HunyuanVideo's attention pre-processing in eager bf16 (teletron/models/hunyuan/model.py:87-125;
+    the two ops are restated from diffusers' published RMSNorm and apply_rotary_emb): per-head RMSNorm
+    on the [B, H, S, D] transposed view, then x * cos + rot(x) * sin in fp32 with real tables [S, D].
+    ``x`` is [B, S, H, D] in memory order, ``freqs_cs`` real [S, D/2, 2].  Returns (y, dx, dgamma)."""
+    cos = freqs_cs[..., 0].repeat_interleave(2, dim=1)
+    sin = freqs_cs[..., 1].repeat_interleave(2, dim=1)
+    mod = EagerRMSNorm(x.shape[-1], eps)
+    mod.weight = nn.Parameter(gamma.detach().clone())
+    xr = x.detach().clone().requires_grad_(True)
+    q = mod(xr.transpose(1, 2))
+    re_, im_ = q.reshape(*q.shape[:-1], -1, 2).unbind(-1)
+    rot = torch.stack([-im_, re_], dim=-1).flatten(3)
+    y = (q.float() * cos + rot.float() * sin).to(q.dtype)
+    y.backward(dy.transpose(1, 2))
+    return y.detach(), xr.grad, mod.weight.grad

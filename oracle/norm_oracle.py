@@ -207,6 +207,27 @@ def rmsnorm_rope_backward(dy, x, gamma, freqs_cs, eps: float, head_dim: int):
     return rmsnorm_backward(rope_apply_backward(dy, freqs_cs, head_dim), x, gamma, eps)
 
 
+def rmsnorm_rope_heads_forward(x, gamma, freqs_cs, eps: float):
+    """HunyuanVideo's per-head QK-norm followed by the rotary embedding
+    (teletron/models/hunyuan/model.py:92-125; the arithmetic of both lives in diffusers >= 0.33.1,
+    which is not vendored: ``RMSNorm`` = x * rsqrt(mean(x^2) + eps) * weight over head_dim, and
+    ``apply_rotary_emb(x, (cos, sin))`` with ``use_real_unbind_dim=-1`` = x * cos + rot(x) * sin with
+    rot(x)[2i] = -x[2i+1], rot(x)[2i+1] = x[2i], i.e. the same pairwise complex rotation as above).
+    ``x`` is [..., S, H, D] in memory order, ``gamma`` [D], ``freqs_cs`` [S, D/2, 2].
+    Returns (y like x, rstd per row)."""
+    y, _, rstd = rmsnorm_forward(x, gamma, eps)
+    d = x.shape[-1]
+    flat = y.reshape(*y.shape[:-2], y.shape[-2] * d)
+    return rope_apply(flat, freqs_cs, d).reshape(y.shape), rstd
+
+
+def rmsnorm_rope_heads_backward(dy, x, gamma, freqs_cs, eps: float):
+    """(dx, dgamma) of the above."""
+    d = x.shape[-1]
+    flat = _f64(dy).reshape(*dy.shape[:-2], dy.shape[-2] * d)
+    return rmsnorm_backward(rope_apply_backward(flat, freqs_cs, d).reshape(dy.shape), x, gamma, eps)
+
+
 # --------------------------------------------------------------------------- gated residual add
 def gate_residual_forward(x, gate, residual, n_batches: int = 1):
     """out = x + gate * residual (teletron/models/wan/wan_model.py:205-210); gate [B, C]."""

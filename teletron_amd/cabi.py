@@ -56,6 +56,10 @@ PROTOTYPES = {
                                         c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_rmsnorm_rope_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                          c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_rmsnorm_rope_heads_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_rmsnorm_rope_heads_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                               c_size_t, c_int64, c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_gate_residual_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "tt_gate_residual_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                           c_int64, c_int64, c_int64, c_void_p]),

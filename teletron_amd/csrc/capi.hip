@@ -71,6 +71,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 struct Rope {
   const float* freqs = nullptr;
   int64_t head_dim = 0, seq_len = 0;
+  int64_t heads = 0;   // 0: a row holds every head of a token; > 0: one head per row, `heads` rows per token
 };
 
 struct Plan {
@@ -105,8 +106,8 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
     if (narrow || kind != kAdaLN || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
     k = res == 2 ? resnorm_gated_kernel(dir == kBwd, idx, full) : resnorm_plain_kernel(dir == kBwd, idx, full);
   } else if (rope) {
-    if (narrow || kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
-    k = rms_rope_kernel(dir == kBwd, idx, full);
+    if (kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
+    k = rms_rope_kernel(narrow, dir == kBwd, idx, full);
   } else if (kind == kAdaLN)
     k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
@@ -189,7 +190,7 @@ size_t workspace_for(int kind, int n_acc, int64_t rows, int64_t cols, int64_t ro
     const size_t ns = partial_bytes(ps, n_acc, cols);
     if (ns > need) need = ns;
   }
-  if (kind == kRMS && cols / kPack > kNarrowMaxPacks) {   // tt_rmsnorm_rope_backward shares this size query
+  if (kind == kRMS) {   // tt_rmsnorm_rope[_heads]_backward share this size query
     Plan pr;
     if (make_plan(kRMS, kBwd, rows, cols, rows, &pr, true) == TT_OK) {
       const size_t nr = partial_bytes(pr, n_acc, cols);
@@ -285,10 +286,16 @@ bool vector_path(int64_t cols, std::initializer_list<const void*> ptrs) {
   return true;
 }
 
-int check_rope(const Rope& rope, int64_t cols) {
-  if (!rope.freqs || rope.head_dim <= 0 || rope.seq_len <= 0) return TT_ERR_INVALID_ARGUMENT;
+int check_rope(const Rope& rope, int64_t rows, int64_t cols) {
+  if (!rope.freqs || rope.head_dim <= 0 || rope.seq_len <= 0 || rope.heads < 0) return TT_ERR_INVALID_ARGUMENT;
   if (rope.head_dim % kPack != 0 || rope.head_dim > 256 || cols % rope.head_dim != 0 || !aligned16(rope.freqs))
     return TT_ERR_UNSUPPORTED;
+  if (rope.heads > 0) {   // one head per row: the narrow kernels
+    if (cols != rope.head_dim) return TT_ERR_UNSUPPORTED;
+    if (rows % rope.heads != 0) return TT_ERR_INVALID_ARGUMENT;
+  } else if (cols / kPack <= kNarrowMaxPacks) {
+    return TT_ERR_UNSUPPORTED;   // all heads in one row: the wide kernels
+  }
   return TT_OK;
 }
 
@@ -298,7 +305,7 @@ int forward(int kind, void* y, const void* x, const void* p0, const void* p1, fl
   if (!y || !x || !p0 || (kind == kAdaLN && !p1)) return TT_ERR_INVALID_ARGUMENT;
   if (rope) {
     if (!vector_path(cols, {y, x, p0})) return TT_ERR_UNSUPPORTED;
-    const int rrc = check_rope(*rope, cols);
+    const int rrc = check_rope(*rope, rows, cols);
     if (rrc != TT_OK) return rrc;
   } else if (!vector_path(cols, {y, x, p0, p1, x_norm})) {
     return forward_generic(kind, y, x, p0, p1, mean, rstd, x_norm, rows, cols, rows_per_batch, eps, stream);
@@ -308,6 +315,7 @@ int forward(int kind, void* y, const void* x, const void* p0, const void* p1, fl
   if (rc != TT_OK) return rc;
   FwdArgs a;
   a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
+  a.rows_per_pos = rope && rope->heads > 0 ? rope->heads : 1;
   a.y = y; a.x = x; a.p0 = p0; a.p1 = p1; a.mean = mean; a.rstd = rstd; a.x_norm = x_norm;
   a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
   a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
@@ -323,7 +331,7 @@ int backward_partials(int kind, void* dx, const void* dy, const void* x, const v
   if (!dx || !dy || !x || !p0) return TT_ERR_INVALID_ARGUMENT;
   if (!aligned16(dx) || !aligned16(dy) || !aligned16(x) || !aligned16(p0)) return TT_ERR_UNSUPPORTED;
   if (rope) {
-    const int rrc = check_rope(*rope, cols);
+    const int rrc = check_rope(*rope, rows, cols);
     if (rrc != TT_OK) return rrc;
   }
   Plan p;
@@ -333,6 +341,7 @@ int backward_partials(int kind, void* dx, const void* dy, const void* x, const v
   if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;
   BwdArgs a;
   a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
+  a.rows_per_pos = rope && rope->heads > 0 ? rope->heads : 1;
   a.dx = dx; a.dy = dy; a.x = x; a.p0 = p0; a.partials = static_cast<float*>(workspace);
   a.rows_per_batch = rows_per_batch; a.n_tiles = p.n_tiles;
   a.cols = (int)cols; a.packs = p.packs; a.eps = eps; a.inv_cols = 1.0f / (float)cols;
@@ -491,6 +500,28 @@ int tt_rmsnorm_rope_backward(void* dx, float* dweight, const void* dy, const voi
                              rows, cols, rows, eps, stream, &rope);
   if (rc != TT_OK) return rc;
   return reduce(dweight, nullptr, workspace, 1, n_partials, 1, cols, false, stream);
+}
+
+int tt_rmsnorm_rope_heads_forward(void* y, const void* x, const void* weight, const float* freqs, float* rstd,
+                                  int64_t rows, int64_t head_dim, int64_t heads, int64_t seq_len, float eps,
+                                  void* stream) {
+  if (heads <= 0) return TT_ERR_INVALID_ARGUMENT;
+  Rope rope; rope.freqs = freqs; rope.head_dim = head_dim; rope.seq_len = seq_len; rope.heads = heads;
+  return forward(kRMS, y, x, weight, nullptr, nullptr, rstd, nullptr, rows, head_dim, rows, eps, stream, &rope);
+}
+
+int tt_rmsnorm_rope_heads_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,
+                                   const float* freqs, void* workspace, size_t workspace_bytes,
+                                   int64_t rows, int64_t head_dim, int64_t heads, int64_t seq_len, float eps,
+                                   void* stream) {
+  if (rows == 0) return TT_OK;
+  if (!dweight || heads <= 0) return TT_ERR_INVALID_ARGUMENT;
+  Rope rope; rope.freqs = freqs; rope.head_dim = head_dim; rope.seq_len = seq_len; rope.heads = heads;
+  int n_partials = 0;
+  int rc = backward_partials(kRMS, dx, dy, x, weight, workspace, workspace_bytes, &n_partials,
+                             rows, head_dim, rows, eps, stream, &rope);
+  if (rc != TT_OK) return rc;
+  return reduce(dweight, nullptr, workspace, 1, n_partials, 1, head_dim, false, stream);
 }
 
 // ---------------------------------------------------------------- gated residual add

@@ -183,7 +183,28 @@ KernelInfo info_bwd_rope_wide() {
   constexpr int R = bwd_wide_R(W, P), Q = bwd_wide_Q(W, P);
   return {reinterpret_cast<const void*>(&norm_bwd_wide<kRMS, W, P, R, Q, FULL, true>), 64 * W * Q, Q * R, P * R};
 }
-inline KernelInfo lookup_rope(bool backward, int idx, bool full) {
+template <int L, bool FULL>
+KernelInfo info_fwd_rope_narrow() {
+  constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&norm_fwd_narrow<kRMS, L, R, NW, FULL, true>), 64 * NW, NW * R * (64 / L), R};
+}
+template <int L, bool FULL>
+KernelInfo info_bwd_rope_narrow() {
+  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  return {reinterpret_cast<const void*>(&norm_bwd_narrow<kRMS, L, R, NW, FULL, true>), 64 * NW, NW * R * (64 / L), R};
+}
+inline KernelInfo lookup_rope(bool narrow, bool backward, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L)                                                                                       \
+  case i:                                                                                             \
+    return backward ? (full ? info_bwd_rope_narrow<L, true>() : info_bwd_rope_narrow<L, false>())     \
+                    : (full ? info_fwd_rope_narrow<L, true>() : info_fwd_rope_narrow<L, false>());
+      TT_NARROW_LIST(X)
+#undef X
+    }
+    return {nullptr, 0, 0, 0};
+  }
   switch (idx) {
 #define X(i, W, P)                                                                                  \
   case i:                                                                                           \
@@ -300,7 +321,7 @@ KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_saved_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
-KernelInfo rms_rope_kernel(bool backward, int idx, bool full);
+KernelInfo rms_rope_kernel(bool narrow, bool backward, int idx, bool full);
 KernelInfo gate_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo gate_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo resnorm_plain_kernel(bool backward, int idx, bool full);

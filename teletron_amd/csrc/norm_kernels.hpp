@@ -49,6 +49,7 @@ struct FwdArgs {
   const float* freqs;
   int64_t seq_len;
   int head_dim;
+  int64_t rows_per_pos;   // narrow ROPE kernels: consecutive rows (heads) that share one position
 };
 
 struct BwdArgs {
@@ -66,6 +67,7 @@ struct BwdArgs {
   const float* freqs;   // as in FwdArgs (ROPE kernels only)
   int64_t seq_len;
   int head_dim;
+  int64_t rows_per_pos;
 };
 
 // Rotary helpers: a pack holds 4 (re, im) pairs; fr holds their 4 (cos, sin) pairs.
@@ -523,12 +525,34 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
   wide_write_partials<ADALN, W, P, Q>(acc0, acc1, act, col, a.partials, b, C, q, w, lane);
 }
 
+// Position of a row for the narrow ROPE kernels: one row is one head, `rows_per_pos` consecutive
+// rows (the heads of a token) share position (row / rows_per_pos) % seq_len.  A lane follows rows
+// row0, row0 + step, row0 + 2 step, ...; the position is kept incrementally (no division in the loop).
+struct RowPos {
+  int64_t head, pos;       // row = (k * seq_len + pos) * rows_per_pos + head
+  int64_t dhead, dpos;     // step = dpos * rows_per_pos + dhead, dpos already reduced mod seq_len
+  __device__ __forceinline__ void init(int64_t row0, int64_t step, int64_t rows_per_pos, int64_t seq_len) {
+    head = row0 % rows_per_pos;
+    pos = (row0 / rows_per_pos) % seq_len;
+    dhead = step % rows_per_pos;
+    dpos = (step / rows_per_pos) % seq_len;
+  }
+  __device__ __forceinline__ void advance(int64_t rows_per_pos, int64_t seq_len) {
+    head += dhead;
+    pos += dpos;
+    if (head >= rows_per_pos) { head -= rows_per_pos; pos += 1; }
+    if (pos >= seq_len) pos -= seq_len;
+    if (pos >= seq_len) pos -= seq_len;
+  }
+};
+
 // ============================================================================ narrow forward
 // L lanes per row (one pack each), 64/L rows per wave per load, R loads in flight,
 // NW independent waves per workgroup.  A tile is NW*R*(64/L) consecutive rows.
-template <int KIND, int L, int R, int NW, bool FULL>
+template <int KIND, int L, int R, int NW, bool FULL, bool ROPE = false>
 __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
+  static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
   constexpr int RPW = 64 / L;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -556,13 +580,30 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   }
 
   u32x4 raw[R];
+  // ROPE: the 4 (cos, sin) pairs of this lane's pack at the row's position travel with the row.
+  float fr[ROPE ? R : 1][8];
+  RowPos rp[ROPE ? R : 1];
+  if constexpr (ROPE) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri + r * RPW,
+                 (int64_t)gridDim.x * (NW * R * RPW), a.rows_per_pos, a.seq_len);
+  }
   auto fetch = [&](int64_t t) {
     const int64_t rb = t * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t rr = rb + r * RPW;
       raw[r] = u32x4{0, 0, 0, 0};
-      if (rr < S && act) raw[r] = load_stream(a.x, (size_t)((b * S + rr) * C + col));
+      if constexpr (ROPE) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) fr[r][j] = 0.f;
+      }
+      if (rr < S && act) {
+        raw[r] = load_stream(a.x, (size_t)((b * S + rr) * C + col));
+        if constexpr (ROPE) load_freq8(a.freqs, (size_t)(rp[r].pos * a.head_dim + col), fr[r]);
+      }
+      if constexpr (ROPE) rp[r].advance(a.rows_per_pos, a.seq_len);
     }
   };
 
@@ -571,12 +612,17 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
     float xf[R][8];
+    float fc[ROPE ? R : 1][8];
     bool rv[R];
     if (!PF) fetch(tile);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       rv[r] = rbase + r * RPW < S;
       unpack8(raw[r], xf[r]);
+      if constexpr (ROPE) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) fc[r][j] = fr[r][j];
+      }
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
 #pragma unroll
@@ -610,6 +656,7 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
           n[j] = xh;
           o[j] = ADALN ? fmaf(xh, g[j], sh[j]) : xh * g[j];
         }
+        if constexpr (ROPE) rope_rotate(o, fc[r]);
         store_stream(a.y, (size_t)(row * C + col), pack8(o));
         if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col), pack8(n));
         if (pi == 0) {
@@ -658,9 +705,10 @@ __device__ __forceinline__ void narrow_write_partials(float (&acc0)[8], float (&
 }
 
 // ============================================================================ narrow backward
-template <int KIND, int L, int R, int NW, bool FULL>
+template <int KIND, int L, int R, int NW, bool FULL, bool ROPE = false>
 __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
+  static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
   constexpr int NACC = ADALN ? 2 : 1;
   constexpr int RPW = 64 / L;
 
@@ -688,6 +736,14 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
   }
 
   u32x4 rawx[R], rawd[R];
+  float fr[ROPE ? R : 1][8];   // as in the forward kernel
+  RowPos rp[ROPE ? R : 1];
+  if constexpr (ROPE) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri + r * RPW,
+                 (int64_t)gridDim.x * (NW * R * RPW), a.rows_per_pos, a.seq_len);
+  }
   auto fetch = [&](int64_t t) {
     const int64_t rb = t * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
 #pragma unroll
@@ -695,11 +751,17 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       const int64_t rr = rb + r * RPW;
       rawx[r] = u32x4{0, 0, 0, 0};
       rawd[r] = u32x4{0, 0, 0, 0};
+      if constexpr (ROPE) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) fr[r][j] = 0.f;
+      }
       if (rr < S && act) {
         const size_t off = (size_t)((b * S + rr) * C + col);
         rawx[r] = load_stream(a.x, off);
         rawd[r] = load_stream(a.dy, off);
+        if constexpr (ROPE) load_freq8(a.freqs, (size_t)(rp[r].pos * a.head_dim + col), fr[r]);
       }
+      if constexpr (ROPE) rp[r].advance(a.rows_per_pos, a.seq_len);
     }
   };
 
@@ -715,6 +777,8 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       rv[r] = rbase + r * RPW < S;
       unpack8(rawx[r], xf[r]);
       unpack8(rawd[r], df[r]);
+      // the incoming gradient is that of the rotated output: undo the rotation first
+      if constexpr (ROPE) rope_unrotate(df[r], fr[r]);
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
     if constexpr (NW > 1) __syncthreads();   // lock-step only: keeps the request stream narrow (+1-2 %)

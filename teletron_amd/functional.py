@@ -105,6 +105,44 @@ class RMSNormRopeFunction(Function):
                 dweight.to(w_dtype).reshape(w_shape) if ctx.needs_input_grad[1] else None, None, None, None)
 
 
+class RMSNormRopeHeadsFunction(Function):
+    """HunyuanVideo's ``apply_rotary_emb(attn.norm_q(query), image_rotary_emb)``
+    (``teletron/models/hunyuan/model.py:92-125``) as one op: ``apply(query, weight, freqs, epsilon)``
+    with ``query`` ``[B, H, S, D]`` as the model holds it (the transposed view of a ``[B, S, H, D]``
+    buffer; processed in memory order without a copy) or ``[B, S, H, D]`` contiguous, ``weight``
+    ``[D]`` and ``freqs`` real ``[S, D/2, 2]`` (cos, sin) or complex ``[S, 1, D/2]`` (no gradient).
+    ``rope_table_from_cos_sin`` converts the model's ``(cos, sin)`` pair."""
+
+    @staticmethod
+    def forward(ctx, x, weight, freqs, epsilon):
+        ctx.eps = float(epsilon)
+        ctx.weight_meta = (weight.shape, weight.dtype)
+        weight_c = weight.detach().to(torch.bfloat16).contiguous()
+        freqs_c = ops._check_freqs(freqs.detach(), x, x.shape[-1])
+        ctx.save_for_backward(x, weight_c, freqs_c)
+        return ops.rmsnorm_rope_heads_forward(x, weight_c, freqs_c, ctx.eps)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight_c, freqs_c = ctx.saved_tensors
+        dx, dweight = ops.rmsnorm_rope_heads_backward(grad_output, x, weight_c, freqs_c, ctx.eps)
+        w_shape, w_dtype = ctx.weight_meta
+        return (dx if ctx.needs_input_grad[0] else None,
+                dweight.to(w_dtype).reshape(w_shape) if ctx.needs_input_grad[1] else None, None, None)
+
+
+def rope_table_from_cos_sin(cos: torch.Tensor, sin: torch.Tensor, extra_tokens: int = 0) -> torch.Tensor:
+    """``(cos, sin)`` tables ``[S, D]`` in which every value appears twice in a row (the
+    ``image_rotary_emb`` pair of HunyuanVideo) -> fp32 ``[S + extra_tokens, D/2, 2]``; the extra
+    tokens (text tokens appended after the latent ones, which take no rotation) get (1, 0)."""
+    table = torch.stack([cos[:, 0::2].float(), sin[:, 0::2].float()], dim=-1)
+    if extra_tokens:
+        ident = torch.zeros(extra_tokens, table.shape[1], 2, dtype=table.dtype, device=table.device)
+        ident[..., 0] = 1.0
+        table = torch.cat([table, ident], dim=0)
+    return table.contiguous()
+
+
 class GateResidualFunction(Function):
     """``x + gate * residual`` with the hand-written backward of ``GateWithGradReduce``
     (``teletron/core/context_parallel/layers.py:24-36``) on one GPU: returns

@@ -270,6 +270,59 @@ def rmsnorm_rope_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tenso
     return dx, dweight
 
 
+def _heads_layout(x: torch.Tensor, weight: torch.Tensor, freqs: torch.Tensor):
+    """x: [..., S, H, D] contiguous or its dense [..., H, S, D] transposed view (the layout HunyuanVideo
+    hands to its per-head norm, teletron/models/hunyuan/model.py:87-95).  Returns the tensor in
+    memory order [..., S, H, D], the permutation that was applied (or None), H, D and S."""
+    _require(isinstance(x, torch.Tensor) and x.dim() >= 3, ValueError, "x must be [..., tokens, heads, head_dim] (or its transposed view)")
+    view, perm = memory_order_view(x)
+    xm = x if view is None else view
+    d = xm.shape[-1]
+    xm = _check_act("x", xm, d)
+    heads, seq = xm.shape[-2], xm.shape[-3]
+    weight = _check_param("weight", weight, xm, d)
+    _require(weight.numel() == d, ValueError, f"weight must have {d} elements, got {weight.numel()}")
+    _require(d % 8 == 0 and d <= 256, ValueError, f"head_dim {d} must be a multiple of 8 and at most 256")
+    freqs = _check_freqs(freqs, xm, d)
+    _require(freqs.shape[0] == seq, ValueError, f"x has {seq} tokens in memory order, freqs {freqs.shape[0]} positions")
+    return xm, perm, weight, freqs, heads, d, seq
+
+
+def rmsnorm_rope_heads_forward(x: torch.Tensor, weight: torch.Tensor, freqs: torch.Tensor, eps: float):
+    """Per-head rope(rmsnorm(x) * weight): every row of head_dim elements is normalised on its own
+    and rotated with the table of its token.  x: [..., S, H, D] bf16 contiguous, or the dense
+    [..., H, S, D] transposed view of such a buffer (processed in memory order without a copy; the
+    result has the input's shape and strides).  freqs: [S, D/2, 2] (cos, sin) or complex [S, 1, D/2]."""
+    xm, perm, weight, freqs, heads, d, seq = _heads_layout(x, weight, freqs)
+    rows = xm.numel() // d
+    y = torch.empty_like(xm)
+    if rows:
+        with torch.cuda.device(xm.device):
+            cabi.call("tt_rmsnorm_rope_heads_forward", y.data_ptr(), xm.data_ptr(), weight.data_ptr(), freqs.data_ptr(),
+                      None, rows, d, heads, seq, float(eps), _stream(xm))
+    return y if perm is None else y.permute(_inverse(perm))
+
+
+def rmsnorm_rope_heads_backward(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, freqs: torch.Tensor, eps: float):
+    """Returns (dx like x, dweight fp32 [D]) for ``rmsnorm_rope_heads_forward``; dy in x's layout."""
+    xm, perm, weight, freqs, heads, d, seq = _heads_layout(x, weight, freqs)
+    _require(isinstance(dy, torch.Tensor) and dy.shape == x.shape and dy.device == x.device, ValueError,
+             "dy must match x in shape and device")
+    dym = dy if perm is None else dy.permute(perm)
+    dym = _check_act("dy", dym, d)          # contiguous copy only if dy is not laid out like x
+    rows = xm.numel() // d
+    dx = torch.empty_like(xm)
+    if rows == 0:
+        return (dx if perm is None else dx.permute(_inverse(perm))), torch.zeros(d, dtype=torch.float32, device=xm.device)
+    dweight = torch.empty(d, dtype=torch.float32, device=xm.device)
+    with torch.cuda.device(xm.device):
+        ws = _workspace(cabi.load().tt_rmsnorm_backward_workspace_bytes(rows, d), 0, xm)
+        cabi.call("tt_rmsnorm_rope_heads_backward", dx.data_ptr(), dweight.data_ptr(), dym.data_ptr(), xm.data_ptr(),
+                  weight.data_ptr(), freqs.data_ptr(), ws.data_ptr(), ws.numel(), rows, d, heads, seq,
+                  float(eps), _stream(xm))
+    return (dx if perm is None else dx.permute(_inverse(perm))), dweight
+
+
 # --------------------------------------------------------------------------- residual update + LayerNorm
 RESIDUAL_NORM_MIN_COLS = 264     # the fused kernels cover rows of more than 256 elements
 

@@ -15,7 +15,7 @@ import torch
 @dataclass(frozen=True)
 class Workload:
     name: str
-    op: str                      # "adaln" | "rmsnorm" | "rope" | "gate" | "resnorm" | "resnorm_gated"
+    op: str                      # "adaln" | "rmsnorm" | "rope" | "rope_heads" | "gate" | "resnorm" | "resnorm_gated"
     shape: Tuple[int, ...]       # activation shape, normalised dim last
     param_shape: Tuple[int, ...]
     eps: float = 1e-6
@@ -45,8 +45,8 @@ class Workload:
         n_param = 1
         for d in self.param_shape:
             n_param *= d
-        if self.op == "rope":        # RMSNorm + rotary embedding: as rmsnorm plus the fp32 (cos, sin) table, read once
-            table = self.shape[-2] * self.head_dim * 4
+        if self.op in ("rope", "rope_heads"):   # RMSNorm + rotary embedding: as rmsnorm plus the fp32 (cos, sin) table, read once
+            table = (self.shape[-2] if self.op == "rope" else self.shape[-3]) * self.head_dim * 4
             fwd = 4 * e + n_param * 2 + table
             bwd = 6 * e + n_param * 2 + n_param * 4 + table
             return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[direction]
@@ -86,6 +86,8 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
              note="the reference's own AdaLN width, through its launcher signatures"),
     Workload("rmsnorm_hunyuan_head_reference_contract", "rmsnorm", (1, 118800, 24, 128), (128,), contract="reference",
              note="the reference's own RMSNorm width, through its launcher signatures"),
+    Workload("rmsnorm_rope_hunyuan_head", "rope_heads", (1, 118800, 24, 128), (128,), head_dim=128,
+             note="HunyuanVideo per-head QK-norm + rotary embedding (per tensor)"),
     Workload("residual_adaln_wan14b", "resnorm", (1, 75600, 5120), (1, 1, 5120),
              note="x + cross_attn(..) fused with norm2 + modulate"),
     Workload("gated_residual_layernorm_wan14b", "resnorm_gated", (1, 75600, 5120), (1, 1, 5120),
@@ -124,12 +126,12 @@ def make_inputs(w: Workload, seed: int = 0, device="cpu", rows: Optional[int] = 
         out["shift"], out["scale"] = shift, scale
     else:
         out["gamma"] = 1.0 + 0.1 * torch.randn(w.param_shape, generator=g, dtype=torch.float32)
-        if w.op == "rope":
-            ang = 3.0 * torch.randn(shape[-2], w.head_dim // 2, generator=g, dtype=torch.float32)
+        if w.op in ("rope", "rope_heads"):
+            ang = 3.0 * torch.randn(shape[-2] if w.op == "rope" else shape[-3], w.head_dim // 2, generator=g, dtype=torch.float32)
             freqs = torch.stack([ang.cos(), ang.sin()], dim=-1)
     dy = torch.randn(shape, generator=g, dtype=torch.float32)
     out["x"], out["dy"] = x, dy
     out = {k: v.to(torch.bfloat16).to(device) for k, v in out.items()}
-    if w.op == "rope":
+    if w.op in ("rope", "rope_heads"):
         out["freqs"] = freqs.to(device)          # fp32 [S, head_dim/2, 2]
     return out

@@ -86,3 +86,93 @@ def test_rope_full_size_rows_and_reproducibility():
     assert_bf16_close(dx[0, di], O.rmsnorm_backward(dyu, x[0, di].cpu(), w.cpu(), 1e-6)[0], "dx via unrotate")
     dx2, dw2 = ops.rmsnorm_rope_backward(dy, x, w, fcs, 1e-6, hd)
     assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
+
+
+# ---------------------------------------------------------------- per-head norm + rotary (HunyuanVideo layout)
+@pytest.mark.parametrize("b,s,heads,hd", [(1, 1, 1, 128), (2, 37, 24, 128), (1, 301, 3, 64), (3, 19, 5, 8), (1, 50, 7, 72),
+                                          (1, 23, 4, 256), (2, 1000, 2, 32)])
+def test_rmsnorm_rope_heads_shapes(b, s, heads, hd):
+    from teletron_amd import ops
+    seed = 1000 + hd + s
+    x, dy = rand_bf16(b, s, heads, hd, seed=seed, scale=1.5), rand_bf16(b, s, heads, hd, seed=seed + 1)
+    w = rand_bf16(hd, seed=seed + 2, scale=0.1, offset=1.0)
+    freqs = make_freqs(s, hd, seed=s)
+    fcs = torch.view_as_real(freqs).reshape(s, hd // 2, 2)
+    y = ops.rmsnorm_rope_heads_forward(x.to(DEV), w.to(DEV), freqs.to(DEV), 1e-6)
+    dx, dw = ops.rmsnorm_rope_heads_backward(dy.to(DEV), x.to(DEV), w.to(DEV), freqs.to(DEV), 1e-6)
+    yo, _ = O.rmsnorm_rope_heads_forward(x, w, fcs, 1e-6)
+    dxo, dwo = O.rmsnorm_rope_heads_backward(dy, x, w, fcs, 1e-6)
+    assert_bf16_close(y, yo, "y")
+    assert_bf16_close(dx, dxo, "dx")
+    assert_grad_close(dw, dwo, b * s * heads, "dweight")
+
+
+def test_rope_heads_function_on_the_transposed_view():
+    """The call pattern of teletron/models/hunyuan/model.py:87-125: query is the [B, H, S, D] transposed
+    view, the rotary tables are real (cos, sin) [S_latent, D] with doubled values, and the text
+    tokens at the end take no rotation."""
+    from teletron_amd import RMSNormModelFunction, RMSNormRopeHeadsFunction, rope_table_from_cos_sin
+    b, s_lat, s_txt, heads, hd = 2, 300, 21, 24, 128
+    s = s_lat + s_txt
+    buf = rand_bf16(b, s, heads * hd, seed=5).to(DEV).requires_grad_(True)
+    dy = rand_bf16(b, heads, s, hd, seed=6).to(DEV)
+    w = rand_bf16(hd, seed=7, scale=0.1, offset=1.0).to(DEV).requires_grad_(True)
+    g = torch.Generator().manual_seed(8)
+    ang = 3.0 * torch.randn(s_lat, hd // 2, generator=g)
+    cos, sin = ang.cos().repeat_interleave(2, dim=1).to(DEV), ang.sin().repeat_interleave(2, dim=1).to(DEV)
+    table = rope_table_from_cos_sin(cos, sin, extra_tokens=s_txt)
+    query = buf.unflatten(2, (heads, -1)).transpose(1, 2)                 # [B, H, S, D] view
+    out = RMSNormRopeHeadsFunction.apply(query, w, table, 1e-6)
+    assert out.shape == query.shape and out.stride() == query.stride()
+    out.backward(dy)
+    x_mem = buf.detach().cpu().reshape(b, s, heads, hd)
+    yo, _ = O.rmsnorm_rope_heads_forward(x_mem, w.detach().cpu(), table.cpu(), 1e-6)
+    dxo, dwo = O.rmsnorm_rope_heads_backward(dy.cpu().transpose(1, 2), x_mem, w.detach().cpu(), table.cpu(), 1e-6)
+    assert_bf16_close(out.transpose(1, 2), yo, "y")
+    assert_bf16_close(buf.grad.reshape(b, s, heads, hd), dxo, "dx")
+    assert_bf16_close(w.grad, dwo, "dweight (bf16 leaf)")
+    # the unrotated tail is bit-identical to the plain fused per-head RMSNorm
+    plain = RMSNormModelFunction.apply(query.detach(), w.detach(), 1e-6, hd)
+    assert torch.equal(out[:, :, s_lat:], plain[:, :, s_lat:])
+    with pytest.raises(ValueError):
+        RMSNormRopeHeadsFunction.apply(query, w, table[:-1], 1e-6)        # positions do not match
+
+
+def test_rope_heads_full_size_whole_tensor():
+    """HunyuanVideo's shape, 118800 tokens x 24 heads x 128: every element against torch fp32 on the GPU."""
+    from teletron_amd import ops
+    from test_gpu_configs import whole_tensor_check
+    s, heads, hd, eps = 118800, 24, 128, 1e-6
+    g = torch.Generator(device=DEV).manual_seed(3)
+    x = torch.randn(1, s, heads, hd, generator=g, device=DEV).to(torch.bfloat16)
+    dy = torch.randn(1, s, heads, hd, generator=g, device=DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(hd, generator=g, device=DEV)).to(torch.bfloat16)
+    ang = 3.0 * torch.randn(s, hd // 2, generator=g, device=DEV)
+    table = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()
+    y = ops.rmsnorm_rope_heads_forward(x, w, table, eps)
+    dx, dw = ops.rmsnorm_rope_heads_backward(dy, x, w, table, eps)
+    fc = torch.view_as_complex(table)                                    # [S, D/2]
+    x2, dy2, y2, dx2 = (t.reshape(s, heads, hd) for t in (x, dy, y, dx))
+    rot = lambda t, f: torch.view_as_real(torch.view_as_complex(t.reshape(*t.shape[:-1], hd // 2, 2).contiguous()) * f[:, None, :]).flatten(-2)
+
+    def parts(r0, r1):
+        xs = x2[r0:r1].float()
+        rstd = torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + eps)
+        return xs * rstd, rstd
+
+    def ref_y(r0, r1):
+        return rot(parts(r0, r1)[0] * w.float(), fc[r0:r1])
+
+    def ref_dx(r0, r1):
+        xh, rstd = parts(r0, r1)
+        gg = rot(dy2[r0:r1].float(), fc[r0:r1].conj()) * w.float()
+        return rstd * (gg - xh * (gg * xh).mean(-1, keepdim=True))
+
+    # blocks of tokens: one row of the check is the 24 heads of a token
+    whole_tensor_check(y.reshape(s, heads * hd), lambda r0, r1: ref_y(r0, r1).reshape(r1 - r0, -1), 4096)
+    whole_tensor_check(dx.reshape(s, heads * hd), lambda r0, r1: ref_dx(r0, r1).reshape(r1 - r0, -1), 4096)
+    acc = torch.zeros(hd, dtype=torch.float64, device=DEV)
+    for r0 in range(0, s, 4096):
+        r1 = min(r0 + 4096, s)
+        acc += (rot(dy2[r0:r1].float(), fc[r0:r1].conj()).double() * parts(r0, r1)[0].double()).sum((0, 1))
+    assert_grad_close(dw, acc.cpu(), s * heads, "dweight")

@@ -247,6 +247,34 @@ def test_rope_matches_complex_arithmetic_and_autograd():
     torch.testing.assert_close(O.rope_apply_backward(O.rope_apply(t0, freqs_cs, d), freqs_cs, d), t0, rtol=1e-12, atol=1e-12)
 
 
+def test_rmsnorm_rope_heads_matches_real_table_form_and_autograd():
+    """Per-head norm + rotary against the real-table formulation that diffusers publishes for
+    apply_rotary_emb (cos / sin tables [S, D] holding each value twice, x * cos + rot(x) * sin) on
+    the [B, H, S, D] layout HunyuanVideo uses, through torch autograd."""
+    b, s, h, d, eps = 2, 5, 3, 16, 1e-6
+    x = rnd(b, s, h, d, seed=80).requires_grad_(True)            # memory order [B, S, H, D]
+    gamma = (1 + rnd(d, seed=81, scale=0.1)).requires_grad_(True)
+    dy = rnd(b, s, h, d, seed=82)
+    ang = rnd(s, d // 2, seed=83, scale=2.0)
+    freqs_cs = torch.stack([ang.cos(), ang.sin()], dim=-1)
+    cos, sin = ang.cos().repeat_interleave(2, dim=1), ang.sin().repeat_interleave(2, dim=1)   # [S, D]
+    q = x.transpose(1, 2)                                         # [B, H, S, D] view, as the model passes it
+    qn = torch.nn.functional.rms_norm(q, (d,), gamma, eps)
+    re_, im_ = qn.reshape(b, h, s, d // 2, 2).unbind(-1)
+    rot = torch.stack([-im_, re_], dim=-1).flatten(3)
+    out = qn * cos + rot * sin
+    out.backward(dy.transpose(1, 2))
+    yo, _ = O.rmsnorm_rope_heads_forward(x, gamma, freqs_cs, eps)
+    torch.testing.assert_close(yo, out.detach().transpose(1, 2), rtol=1e-12, atol=1e-12)
+    dxo, dgo = O.rmsnorm_rope_heads_backward(dy, x, gamma, freqs_cs, eps)
+    torch.testing.assert_close(dxo, x.grad, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(dgo, gamma.grad, rtol=1e-10, atol=1e-12)
+    # (cos, sin) = (1, 0) leaves the normalised value alone: tokens that take no rotation
+    ident = torch.stack([torch.ones(s, d // 2), torch.zeros(s, d // 2)], dim=-1)
+    torch.testing.assert_close(O.rmsnorm_rope_heads_forward(x, gamma, ident, eps)[0],
+                               O.rmsnorm_forward(x, gamma, eps)[0], rtol=0, atol=0)
+
+
 def test_gate_residual_matches_autograd():
     nb, s, c = 3, 5, 24
     x, r, dy = rnd(nb, s, c, seed=50).requires_grad_(True), rnd(nb, s, c, seed=51).requires_grad_(True), rnd(nb, s, c, seed=52)
