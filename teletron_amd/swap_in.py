@@ -28,6 +28,9 @@ ships no code that performs the swap.  This module does it by patching *instance
   self-attention update with the affine ``norm3``, and the cross-attention update with
   ``norm2`` + modulate (:func:`fused_dit_block_forward`); 24 instead of 30 bytes per element move
   through HBM for the block's residual/normalisation work in forward, 40 instead of 60 in backward.
+  Every ``SelfAttention`` (``wan_model.py:136-160``) gets a ``forward`` that runs ``norm_q`` /
+  ``norm_k`` and the ``rope_apply`` after them as one kernel per tensor
+  (:func:`fused_self_attention_forward`).
 
 Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` / ``gate_with_cp_grad_reduce``
 all-reduce their parameter gradients over the context-parallel group
@@ -44,8 +47,9 @@ from typing import Callable, Iterable, Optional
 import torch
 import torch.nn as nn
 
-from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, adaln_modulate,
-                         residual_adaln, residual_layer_norm)
+from . import ops
+from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, RMSNormRopeFunction,
+                         adaln_modulate, residual_adaln, residual_layer_norm)
 
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
@@ -194,6 +198,26 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
     return GateResidualFunction.apply(x, gate_mlp, self.ffn(input_x))
 
 
+def fused_self_attention_forward(self, x, freqs):
+    """``SelfAttention.forward`` (``wan_model.py:153-160``) with ``norm_q`` / ``norm_k`` and the
+    ``rope_apply`` that follows each of them in one kernel per tensor; projections and the attention
+    module (possibly wrapped for context parallelism) are used as they are."""
+    q, k = self.q(x), self.k(x)
+    head_dim = q.shape[-1] // self.num_heads
+    if not (q.is_cuda and q.dtype == torch.bfloat16 and q.shape[-1] > 256 and head_dim % 8 == 0 and head_dim <= 256
+            and q.dim() >= 2 and freqs.shape[0] == q.shape[-2]):
+        return type(self).forward(self, x, freqs)
+    table = ops._check_freqs(freqs.detach(), q, head_dim)          # converted once, shared by q and k
+    q = RMSNormRopeFunction.apply(q, self.norm_q.weight, table, self.norm_q.eps, self.num_heads)
+    k = RMSNormRopeFunction.apply(k, self.norm_k.weight, table, self.norm_k.eps, self.num_heads)
+    return self.o(self.attn(q, k, self.v(x)))
+
+
+def _is_self_attention(m: nn.Module) -> bool:
+    return (type(m).__name__ == "SelfAttention" and all(hasattr(m, a) for a in ("q", "k", "v", "o", "attn", "num_heads"))
+            and _is_rmsnorm(getattr(m, "norm_q", None)) and _is_rmsnorm(getattr(m, "norm_k", None)))
+
+
 def _is_dit_block(m: nn.Module) -> bool:
     if type(m).__name__ not in BLOCK_CLASSES:
         return False
@@ -209,7 +233,7 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
     ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
     tokens.  ``blocks`` also replaces the forward of whole DiT blocks (see the module docstring).
     Returns counts of what was swapped."""
-    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0}
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0, "attention": 0}
     for ns in namespaces:
         fn = getattr(ns, "modulate", None)
         if callable(fn) and not hasattr(fn, "__wrapped__"):
@@ -226,6 +250,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_dit_block_forward, module)
             counts["block"] += 1
+        if blocks and rmsnorm and _is_self_attention(module) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(fused_self_attention_forward, module)
+            counts["attention"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
             # The *_with_cp_grad_reduce callables all-reduce their parameter gradients over the
             # context-parallel group; they are only replaced where that is the identity.  An owner

@@ -143,7 +143,7 @@ def test_swap_in_matches_eager_model(monkeypatch):
     assert S.swap_in_if_requested(model, [ns]) is None
     monkeypatch.setenv("FUSED_KERNELS", "1")
     counts = S.swap_in_if_requested(model, [ns])
-    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4, "block": 0}, counts
+    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4, "block": 0, "attention": 0}, counts
     assert isinstance(model.blocks[0].norm3, nn.LayerNorm)               # affine LayerNorm untouched
     assert list(model.state_dict().keys()) == keys_before                 # checkpoint compatible
     try:
@@ -157,7 +157,7 @@ def test_swap_in_matches_eager_model(monkeypatch):
         assert rel(a, b) < 2e-2
     worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
     assert worst < 2e-2, worst
-    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0, "block": 0}   # idempotent on the model
+    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0, "block": 0, "attention": 0}   # idempotent on the model
 
 
 class RefAttention(nn.Module):
@@ -234,6 +234,65 @@ def test_block_level_swap_in_matches_eager_block(dim):
     assert rel(out_f, out_e) < 5e-3
     for a, b in zip(gin_f, gin_e):
         assert rel(a, b) < 2e-2
+    worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
+    assert worst < 2e-2, worst
+
+
+def rope_apply(x, freqs, num_heads):
+    """The model's own rotary embedding (wan_model.py:105-110), restated for the stand-in."""
+    b, s, c = x.shape
+    x_out = torch.view_as_complex(x.to(torch.float64).reshape(b, s, num_heads, -1, 2))
+    return torch.view_as_real(x_out * freqs).flatten(2).to(x.dtype)
+
+
+class SelfAttention(nn.Module):
+    """Attributes and forward of wan_model.py:136-160; the attention core is a stand-in."""
+
+    def __init__(self, dim, num_heads, eps=1e-6):
+        super().__init__()
+        self.num_heads = num_heads
+        self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
+        self.norm_q, self.norm_k = RMSNorm(dim, eps), RMSNorm(dim, eps)
+        self.attn = lambda q, k, v: torch.tanh(q) * k + v
+
+    def forward(self, x, freqs):
+        q = self.norm_q(self.q(x))
+        k = self.norm_k(self.k(x))
+        v = self.v(x)
+        q = rope_apply(q, freqs, self.num_heads)
+        k = rope_apply(k, freqs, self.num_heads)
+        return self.o(self.attn(q, k, v))
+
+
+def test_self_attention_swap_in_fuses_norm_and_rope():
+    from teletron_amd import swap_in as S
+    torch.manual_seed(5)
+    dim, heads, bsz, seq = 512, 4, 2, 75
+    attn = SelfAttention(dim, heads).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        attn.norm_q.weight.add_(0.1 * torch.randn_like(attn.norm_q.weight))
+        attn.norm_k.weight.add_(0.1 * torch.randn_like(attn.norm_k.weight))
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(bsz, seq, dim, generator=g).to(torch.bfloat16).to(DEV)
+    dy = torch.randn(bsz, seq, dim, generator=g).to(torch.bfloat16).to(DEV)
+    ang = 3.0 * torch.randn(seq, dim // heads // 2, generator=g, dtype=torch.float64)
+    freqs = torch.polar(torch.ones_like(ang), ang).reshape(seq, 1, -1).to(DEV)       # complex128, as precompute_freqs_cis
+
+    class Wrap(nn.Module):
+        def __init__(self, m):
+            super().__init__()
+            self.self_attn = m
+
+        def forward(self, x):
+            return self.self_attn(x, freqs)
+
+    model = Wrap(attn)
+    out_e, gin_e, gp_e = run(model, [x], dy)
+    counts = S.swap_in(model, blocks=True)
+    assert counts["attention"] == 1 and counts["rmsnorm"] == 2, counts
+    out_f, gin_f, gp_f = run(model, [x], dy)
+    assert rel(out_f, out_e) < 5e-3
+    assert rel(gin_f[0], gin_e[0]) < 2e-2
     worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
     assert worst < 2e-2, worst
 

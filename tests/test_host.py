@@ -154,7 +154,7 @@ def test_swap_in_leaves_context_parallel_callables_alone_with_several_ranks(monk
     monkeypatch.setattr(S, "_several_ranks", lambda: True)
     many = make()
     counts = S.swap_in(many, blocks=True)
-    assert counts["modulate"] == 0 and counts["gate"] == 0 and counts["block"] == 0 and counts["layernorm"] == 0
+    assert counts["modulate"] == 0 and counts["gate"] == 0 and counts["block"] == 0 and counts["layernorm"] == 0 and counts["attention"] == 0
     assert isinstance(many.norm1, nn.LayerNorm)
     assert not hasattr(many.modulate_with_cp_grad_reduce, "__wrapped__")
     assert "forward" not in many.__dict__
