@@ -51,6 +51,9 @@ def parse_args():
                                       "residual_adaln_wan14b,gated_residual_layernorm_wan14b,rmsnorm_rope_hunyuan_head",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--no-eager-gpu", action="store_true", help="skip timing the eager PyTorch expressions on the GPU")
+    ap.add_argument("--block-demo", action="store_true",
+                    help="also time a whole DiT-block stand-in (Wan2.1-1.3B and 14B widths, 32760 tokens) in eager "
+                         "PyTorch and after swap_in(blocks=True)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
                          "that hardware byte counters collected over this run can be scaled against it")
@@ -312,6 +315,105 @@ def eager_gpu(w, iters=5):
     return (time.perf_counter() - t0) / iters * 1e3
 
 
+def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3):
+    """Whole-block view (--block-demo): a stand-in with the structure of Wan's DiTBlock
+    (teletron/models/wan/wan_model.py:126-244: nn.Linear projections, torch SDPA as the attention
+    core, tanh-GELU FFN) timed forward + backward in eager PyTorch and again after
+    swap_in(blocks=True).  The GEMMs and the attention dominate; this shows what the fused
+    normalisation / residual kernels are worth inside a block."""
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    from teletron_amd import swap_in as S
+    dev, bf = "cuda:0", torch.bfloat16
+
+    def rope_apply(x, freqs, n):
+        b, s, c = x.shape
+        xc = torch.view_as_complex(x.to(torch.float64).reshape(b, s, n, -1, 2))
+        return torch.view_as_real(xc * freqs).flatten(2).to(x.dtype)
+
+    class RMSNorm(nn.Module):
+        def __init__(self, d, eps):
+            super().__init__()
+            self.eps, self.weight = eps, nn.Parameter(torch.ones(d))
+
+        def forward(self, x):
+            xf = x.float()
+            return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)).to(x.dtype) * self.weight
+
+    class AttentionModule(nn.Module):
+        def forward(self, q, k, v):
+            b, s, c = q.shape
+            sh = lambda t: t.reshape(b, t.shape[1], heads, -1).transpose(1, 2)
+            return F.scaled_dot_product_attention(sh(q), sh(k), sh(v)).transpose(1, 2).reshape(b, s, c)
+
+    class SelfAttention(nn.Module):
+        def __init__(self, cross=False):
+            super().__init__()
+            self.num_heads, self.cross = heads, cross
+            self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
+            self.norm_q, self.norm_k, self.attn = RMSNorm(dim, 1e-6), RMSNorm(dim, 1e-6), AttentionModule()
+
+        def forward(self, x, other):
+            src = other if self.cross else x
+            q, k, v = self.norm_q(self.q(x)), self.norm_k(self.k(src)), self.v(src)
+            if not self.cross:
+                q, k = rope_apply(q, other, heads), rope_apply(k, other, heads)
+            return self.o(self.attn(q, k, v))
+
+    class CrossAttention(SelfAttention):
+        def __init__(self):
+            super().__init__(cross=True)
+
+    class GateModule(nn.Module):
+        def forward(self, x, gate, residual):
+            return x + gate * residual
+
+    class DiTBlock(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.self_attn, self.cross_attn = SelfAttention(), CrossAttention()
+            self.norm1 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
+            self.norm2 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
+            self.norm3 = nn.LayerNorm(dim, eps=1e-6)
+            self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate="tanh"), nn.Linear(ffn_dim, dim))
+            self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
+            self.gate, self.gate2 = GateModule(), GateModule()
+
+        def forward(self, x, context, t_mod, freqs):
+            sh1, sc1, g1, sh2, sc2, g2 = (self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
+            x = self.gate(x, g1, self.self_attn(self.norm1(x) * (1 + sc1) + sh1, freqs))
+            x = x + self.cross_attn(self.norm3(x), context)
+            return self.gate2(x, g2, self.ffn(self.norm2(x) * (1 + sc2) + sh2))
+
+    torch.manual_seed(0)
+    blk = DiTBlock().to(dev).to(bf)
+    x = torch.randn(1, seq, dim, device=dev, dtype=bf, requires_grad=True)
+    ctx, dy = torch.randn(1, ctx_len, dim, device=dev, dtype=bf), torch.randn(1, seq, dim, device=dev, dtype=bf)
+    t_mod = 0.2 * torch.randn(1, 6, dim, device=dev, dtype=bf)
+    ang = torch.randn(seq, dim // heads // 2, dtype=torch.float64)
+    freqs = torch.polar(torch.ones_like(ang), ang).reshape(seq, 1, -1).to(dev)
+
+    def timed():
+        for i in range(2 + iters):
+            if i == 2:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            blk(x, ctx, t_mod, freqs).backward(dy)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e3
+
+    eager_ms = timed()
+    out_e = blk(x, ctx, t_mod, freqs).detach()
+    counts = S.swap_in(blk, blocks=True)
+    fused_ms = timed()
+    out_f = blk(x, ctx, t_mod, freqs).detach()
+    diff = float((out_f.double() - out_e.double()).norm() / out_e.double().norm())
+    return {"block": f"DiTBlock stand-in, dim {dim}, {heads} heads, ffn {ffn_dim}, x[1,{seq},{dim}] bf16, context {ctx_len}",
+            "eager_ms": round(eager_ms, 2), "fused_ms": round(fused_ms, 2), "speedup": round(eager_ms / fused_ms, 3),
+            "relative_output_difference": diff, "swapped": counts}
+
+
 def cpu_baseline(w, seconds):
     """PyTorch-eager fwd + autograd bwd of the same op on the host CPU, bounded row sample."""
     import torch
@@ -430,6 +532,8 @@ def main():
                 also[name]["speedup_vs_eager_gpu"] = round(ms / ra["ms_per_step"], 2)
     if also:
         out["also"] = also
+    if args.block_demo:
+        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824)]
     if args.calibrate_copy:
         src = torch.empty(w.elements, dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
         dst = torch.empty_like(src)
