@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E peak
 # known size); the counters cannot be read from inside this process, so the measured figures are
 # carried here.  Valid only while the backward kernel writes the stated number of partial sums.
 MEASURED_TRAFFIC_BYTES = {
-    "adaln_wan14b": {"fwd": 1548486757, "bwd": 2332779792, "n_partials": 248},
+    "adaln_wan14b": {"fwd": 1548486725, "bwd": 2332780526, "n_partials": 248},
 }
 METRIC = "fwd+bwd HBM GB/s and % of peak, AdaLN/RMSNorm at Wan-14B shape 75600x5120"
 
