@@ -387,6 +387,69 @@ def test_golden_fixture(path):
         np.testing.assert_allclose(d["rstd"], rstd.numpy(), rtol=1e-12, atol=0)
 
 
+@pytest.mark.parametrize("path", __import__("fused_fixtures").FUSED, ids=os.path.basename)
+def test_fused_golden_fixture(path):
+    """Fixtures of the ops around the normalisations: the oracle reproduces the stored outputs, and
+    torch autograd on the unfused float64 expression (library layer_norm / rms_norm, complex
+    multiplication for the rotary embedding) reaches them by an independent route."""
+    import fused_fixtures as FF
+    t = FF.load(path)
+    op, eps = t["op"], t["eps"]
+    leaf = lambda v: v.double().clone().requires_grad_(True)
+    if op == "gate":
+        nb = t["x"].shape[0]
+        got = dict(zip(FF.OUTPUTS[op], (O.gate_residual_forward(t["x"], t["gate"], t["residual"], nb),)
+                       + O.gate_residual_backward(t["dy"], t["gate"], t["residual"], nb)[1:]))
+        x, g, r = leaf(t["x"]), leaf(t["gate"]), leaf(t["residual"])
+        out = x + g * r
+        out.backward(t["dy"].double())
+        ref = {"out": out.detach(), "dgate": g.grad.reshape(nb, -1), "dresidual": r.grad}
+    elif op in ("rope", "rope_heads"):
+        x, gamma, f = leaf(t["x"]), leaf(t["gamma"]), t["freqs"].double()
+        fc = torch.view_as_complex(f.contiguous())                               # [S, hd/2]
+        if op == "rope":
+            hd = t["head_dim"]
+            got = dict(zip(FF.OUTPUTS[op], (O.rmsnorm_rope_forward(t["x"], t["gamma"], t["freqs"], eps, hd)[0],)
+                           + O.rmsnorm_rope_backward(t["dy"], t["x"], t["gamma"], t["freqs"], eps, hd)))
+            yn = F.rms_norm(x, (x.shape[-1],), weight=gamma, eps=eps)
+            b, s_, c = yn.shape
+            y = torch.view_as_real(torch.view_as_complex(yn.reshape(b, s_, c // hd, hd // 2, 2)) * fc[None, :, None, :]).reshape(b, s_, c)
+        else:
+            got = dict(zip(FF.OUTPUTS[op], (O.rmsnorm_rope_heads_forward(t["x"], t["gamma"], t["freqs"], eps)[0],)
+                           + O.rmsnorm_rope_heads_backward(t["dy"], t["x"], t["gamma"], t["freqs"], eps)))
+            yn = F.rms_norm(x, (x.shape[-1],), weight=gamma, eps=eps)              # [B, S, H, D]
+            y = torch.view_as_real(torch.view_as_complex(yn.reshape(*yn.shape[:-1], -1, 2)) * fc[None, :, None, :]).reshape(yn.shape)
+        y.backward(t["dy"].double())
+        ref = {"y": y.detach(), "dx": x.grad, "dgamma": gamma.grad}
+    else:
+        affine, gate = bool(t["affine"]), t.get("gate")
+        nb, c = t["x"].shape[0], t["x"].shape[-1]
+        s_o, y_o = O.residual_norm_forward(t["x"], t["residual"], gate, t["scale"], t["shift"], eps, nb, affine)
+        back = O.residual_norm_backward(t["dy"], t["ds_in"], s_o, t["residual"], gate, t["scale"], eps, nb, affine)
+        got = {"s": s_o, "y": y_o, "dx": back[0], "dresidual": back[1], "dscale": back[2], "dshift": back[3], "dgate": back[4]}
+        # independent route: the stored (bf16-rounded) s is a leaf that collects both gradients
+        sl, sc, sh = leaf(t["s"]), leaf(t["scale"]), leaf(t["shift"])
+        if affine:
+            y = F.layer_norm(sl, (c,), sc.reshape(-1), sh.reshape(-1), eps)
+        else:
+            y = F.layer_norm(sl, (c,), None, None, eps) * (1 + sc[:, None, :]) + sh[:, None, :]
+        torch.autograd.backward([y, sl], [t["dy"].double(), t["ds_in"].double()])
+        ref = {"y": y.detach(), "dx": sl.grad, "dscale": sc.grad if not affine else None, "dshift": sh.grad if not affine else None}
+        unrounded = t["x"].double() + (gate.double()[:, None, :] * t["residual"].double() if gate is not None else t["residual"].double())
+        ref["s"] = unrounded.bfloat16().double()
+        if affine:      # stored per batch; the shared parameter's gradient is their sum
+            torch.testing.assert_close(t["dscale"].sum(0, keepdim=True), sc.grad, rtol=1e-9, atol=1e-10)
+            torch.testing.assert_close(t["dshift"].sum(0, keepdim=True), sh.grad, rtol=1e-9, atol=1e-10)
+        if gate is not None:
+            ref["dresidual"] = gate.double()[:, None, :] * sl.grad
+            ref["dgate"] = (sl.grad * t["residual"].double()).sum(1)
+    for name in FF.OUTPUTS[op]:
+        np.testing.assert_allclose(t[name].numpy(), got[name].numpy(), rtol=1e-12, atol=1e-12, err_msg=name)
+        if ref.get(name) is not None:
+            np.testing.assert_allclose(t[name].numpy(), ref[name].reshape(t[name].shape).numpy(), rtol=1e-9, atol=1e-10,
+                                       err_msg=name + " vs autograd")
+
+
 # ------------------------------------------------------------------ eager bf16 restatement (the CPU baseline) vs oracle
 def test_eager_modules_agree_with_oracle_within_bf16():
     g = torch.Generator().manual_seed(31)
