@@ -158,3 +158,30 @@ def test_residual_norm_full_size(name):
     assert_grad_close(dshift, acc[1].cpu(), w.rows, "dshift")
     if gated:
         assert_grad_close(dgate / 2, acc[2].cpu() / 2, w.rows, "dgate")
+
+
+def test_residual_norm_special_cases():
+    """Closed forms: a zero gate passes x through bit for bit; a residual that cancels x gives
+    constant (zero) rows, whose normalised value is 0, so y is the shift itself and every
+    gradient stays finite."""
+    from teletron_amd import ops
+    nb, rpb, cols = 2, 37, 1536
+    x, r, dy, dsi = (rand_bf16(nb, rpb, cols, seed=70 + i).to(DEV) for i in range(4))
+    scale, shift = (rand_bf16(nb, cols, seed=75 + i, scale=0.3).to(DEV) for i in range(2))
+    zero_gate = torch.zeros(nb, cols, dtype=torch.bfloat16, device=DEV)
+    s, y = ops.residual_norm_forward(x, r, zero_gate, scale, shift, 1e-6)
+    assert torch.equal(s, x)
+    assert torch.equal(y, ops.adaln_forward(x, scale, shift, 1e-6))
+    dx, dr, dscale, dshift, dgate = ops.residual_norm_backward(dy, dsi, s, r, zero_gate, scale, 1e-6)
+    assert torch.count_nonzero(dr) == 0
+    dx_ref, dscale_ref, dshift_ref = ops.adaln_backward(dy, x, scale, 1e-6)
+    assert_bf16_close(dx, dsi.double().cpu() + dx_ref.double().cpu(), "dx = ds_in + dAdaLN")
+    assert_grad_close(dscale, dscale_ref.double().cpu(), rpb, "dscale")      # same sums, different summation order
+    assert_grad_close(dshift, dshift_ref.double().cpu(), rpb, "dshift")
+
+    s0, y0 = ops.residual_norm_forward(x, -x, None, scale, shift, 1e-6)
+    assert torch.count_nonzero(s0) == 0
+    assert torch.equal(y0, shift[:, None, :].expand(nb, rpb, cols))
+    out = ops.residual_norm_backward(dy, dsi, s0, None, None, scale, 1e-6)
+    assert all(torch.isfinite(t.float()).all() for t in out if t is not None)
+    assert torch.count_nonzero(out[2]) == 0            # dscale = sum dy * x_hat with x_hat = 0
