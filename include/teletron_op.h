@@ -62,7 +62,7 @@ TT_API int tt_last_hip_error(void);
 /* ------------------------------------------------------------------ fused AdaLN
  * y = LayerNorm_noaffine(x) * (1 + scale) + shift
  *
- * Replaces launch_adaln_forward (teletron_op/fused_adaln/include/adaln_kernel.h:21-30,
+ * Replaces launch_adaln_forward (teletron_op/fused_adaln/include/adaln_kernel.h:20-29,
  * teletron_op/fused_adaln/adaln_forward.cu:198-220) for any `cols`, with
  * per-sample modulation: scale/shift are [n_batches, cols] bf16 where row r uses
  * batch r / rows_per_batch (pass rows_per_batch = rows for a single [cols] vector,
@@ -75,7 +75,7 @@ TT_API int tt_adaln_forward(void* y, const void* x, const void* scale, const voi
                      float eps, void* stream);
 
 /* Backward of the above.  Replaces launch_adaln_backward + launch_adaln_scale_shift_backward
- * (adaln_kernel.h:32-46, adaln_backward.cu:129-151, scale_shift_backward.cu:129-147):
+ * (adaln_kernel.h:31-44, adaln_backward.cu:129-151, scale_shift_backward.cu:129-147):
  *   g = dy * (1 + scale);  dx = rstd * (g - mean(g) - x_hat * mean(g * x_hat))
  *   dscale[b, c] = sum_{rows of batch b} dy * x_hat;  dshift[b, c] = sum dy
  * Inputs dy, x: [rows, cols] bf16; scale: [n_batches, cols] bf16.
@@ -254,12 +254,12 @@ TT_API int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes
  * reduced in fp32 before the single rounding to bf16.
  */
 
-/* launch_adaln_forward: adaln_kernel.h:21-30, adaln_forward.cu:198-220, called from adaln_ops.cpp:16-26. */
+/* launch_adaln_forward: adaln_kernel.h:20-29, adaln_forward.cu:198-220, called from adaln_ops.cpp:16-26. */
 TT_API int tt_launch_adaln_forward(void* output, void* x_norm, const void* input,
                                    const void* scale, const void* shift,
                                    int64_t rows, int64_t cols, double epsilon,
                                    float* inv_variance, void* stream);
-/* launch_adaln_backward: adaln_kernel.h:37-46, adaln_backward.cu:129-151, called from adaln_ops.cpp:39-49.
+/* launch_adaln_backward: adaln_kernel.h:36-44, adaln_backward.cu:129-151, called from adaln_ops.cpp:39-49.
  * Workspace: tt_adaln_backward_workspace_bytes(rows, cols, rows). */
 TT_API int tt_launch_adaln_backward(void* dinp, void* dscale, void* dshift,
                                     const void* dout, const void* x_norm, const void* scale,
