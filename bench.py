@@ -303,6 +303,32 @@ def eager_gpu(w, iters=5):
             else:                     # residual add + norm2 + modulate
                 y = F.layer_norm(s, (c,), eps=w.eps) * (1 + scale) + shift
             torch.autograd.backward([y, s], [dy, ds_in])
+    elif w.op in ("rope", "rope_heads"):
+        weight = rnd(c, scale=0.1, offset=1.0).requires_grad_(True)
+        seq = shape[-2] if w.op == "rope" else shape[-3]
+        ang = 3.0 * torch.randn(seq, w.head_dim // 2, generator=g, device=dev, dtype=torch.float64)
+
+        def rms(t):
+            tf = t.float()
+            return (tf * torch.rsqrt(tf.pow(2).mean(dim=-1, keepdim=True) + w.eps)).to(bf) * weight
+
+        if w.op == "rope":       # norm_q + rope_apply (wan_model.py:105-110,154-157): float64 complex multiply
+            freqs = torch.polar(torch.ones_like(ang), ang).reshape(seq, 1, -1)
+            heads = c // w.head_dim
+
+            def fn():
+                q = rms(x)
+                qc = torch.view_as_complex(q.to(torch.float64).reshape(q.shape[0], seq, heads, -1, 2))
+                torch.view_as_real(qc * freqs).flatten(2).to(bf).backward(dy)
+        else:                    # per-head norm on the [B,H,S,D] view + real-table rotary (hunyuan/model.py:87-125)
+            cos = ang.cos().float().repeat_interleave(2, dim=1)
+            sin = ang.sin().float().repeat_interleave(2, dim=1)
+
+            def fn():
+                q = rms(x.transpose(1, 2))
+                re_, im_ = q.reshape(*q.shape[:-1], -1, 2).unbind(-1)
+                rot = torch.stack([-im_, re_], dim=-1).flatten(3)
+                (q.float() * cos + rot.float() * sin).to(bf).backward(dy.transpose(1, 2))
     else:
         return None
     for _ in range(2):
