@@ -59,6 +59,22 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.tt_adaln_backward(None, None, None, None, None, None, None, 0, 0, 64, 1, 1e-6, None) == cabi.TT_OK
     with pytest.raises(cabi.TeletronOpError):
         cabi.call("tt_rmsnorm_forward", None, p16, p16, None, 4, 64, 1e-6, None)
+    # the fused neighbours validate the same way
+    INV, UNS, OK = cabi.TT_ERR_INVALID_ARGUMENT, cabi.TT_ERR_UNSUPPORTED, cabi.TT_OK
+    assert lib.tt_residual_norm_forward(p16, p16, p16, None, None, 1, p16, p16, 1, 0, None, None, 4, 512, 4, 1e-6, None) == INV
+    assert lib.tt_residual_norm_forward(p16, p16, p16, p16, None, 1, p16, p16, 1, 0, None, None, 4, 516, 4, 1e-6, None) == UNS
+    assert lib.tt_residual_norm_forward(None, None, None, None, None, 1, None, None, 1, 0, None, None, 0, 512, 1, 1e-6, None) == OK
+    assert lib.tt_residual_norm_backward(p16, None, p16, p16, None, p16, None, p16, None, p16, 1, p16, 1, 0,
+                                         p16, 64, 4, 512, 4, 1e-6, None) == INV      # a gate without dr / dgate / r
+    assert lib.tt_residual_norm_backward_workspace_bytes(4, 516, 4, 0) == 0
+    assert lib.tt_gate_residual_forward(p16, p16, None, p16, 4, 64, 4, None) == INV
+    assert lib.tt_gate_residual_forward(p16, p16, p16, p16 + 2, 4, 64, 4, None) == UNS
+    assert lib.tt_rmsnorm_rope_heads_forward(p16, p16, p16, p16, None, 4, 64, 0, 2, 1e-6, None) == INV   # heads <= 0
+    assert lib.tt_rmsnorm_rope_heads_forward(p16, p16, p16, None, None, 4, 64, 2, 2, 1e-6, None) == INV  # no table
+    assert lib.tt_rmsnorm_rope_heads_forward(p16, p16, p16, p16, None, 5, 64, 2, 2, 1e-6, None) == INV   # rows % heads
+    assert lib.tt_rmsnorm_rope_heads_forward(p16, p16, p16, p16, None, 4, 512, 2, 2, 1e-6, None) == UNS  # head_dim > 256
+    assert lib.tt_rmsnorm_rope_forward(p16, p16, p16, p16, None, 4, 128, 64, 4, 1e-6, None) == UNS       # all heads in a short row
+    assert lib.tt_stream_probe(p16, p16, None, 24, None) == UNS and lib.tt_stream_probe(None, None, None, 0, None) == OK
 
 
 def test_python_validation_on_cpu_tensors():
