@@ -411,11 +411,13 @@ const char* tt_error_string(int code) {
 
 int tt_last_hip_error(void) { return g_last_hip_error; }
 
-// Tuning hook (not part of the public header): force the number of resident
-// workgroups per CU that launch plans assume; 0 restores the occupancy query.
+#ifdef TT_TUNING_HOOKS
+// Tuning hooks, compiled only into sweep builds (not part of the public header): force the number
+// of resident workgroups per CU that launch plans assume, or the total number of workgroups of a
+// launch; 0 restores the plan's own choice.
 TT_API void tt_debug_set_wgs_per_cu(int n) { g_wgs_per_cu_override.store(n < 0 ? 0 : n); }
-// Tuning hook: force the total number of workgroups of a launch (0 = off).
 TT_API void tt_debug_set_grid(int n) { g_grid_override.store(n < 0 ? 0 : n); }
+#endif
 
 int tt_adaln_forward(void* y, const void* x, const void* scale, const void* shift, float* mean, float* rstd,
                      int64_t rows, int64_t cols, int64_t rows_per_batch, float eps, void* stream) {
