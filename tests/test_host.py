@@ -25,6 +25,11 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(lib, n), f"{n} declared in include/ but not exported"
     from teletron_amd import cabi
     assert set(cabi.PROTOTYPES) == names, "ctypes prototypes and header disagree"
+    # and nothing else: the dynamic symbol table holds no undeclared entry point
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", str(cabi.LIB_PATH)], capture_output=True, text=True, check=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    assert {n for n in exported if n.startswith("tt_")} == names
 
 
 def test_version_and_error_strings(lib):
