@@ -27,8 +27,9 @@
  * tt_error_string() maps a code to text and tt_last_hip_error() returns the
  * hipError_t recorded by the calling thread's last TT_ERR_HIP.  Kernels are
  * enqueued on `stream` (NULL = the default stream) of the *current* device and
- * the calls do not synchronise.  The library keeps no mutable global state, so
- * calls from several host threads on different streams are safe.
+ * the calls do not synchronise.  Apart from tt_adaln_backward_static (which says so) the
+ * library keeps no mutable device state, so calls from several host threads on different
+ * streams are safe.
  */
 #ifndef TELETRON_OP_H_
 #define TELETRON_OP_H_
@@ -51,6 +52,7 @@ extern "C" {
 #define TT_ERR_UNSUPPORTED 2       /* shape outside what the entry point covers (see above; cols > TT_MAX_COLS) */
 #define TT_ERR_WORKSPACE 3         /* workspace pointer null or smaller than *_workspace_bytes() */
 #define TT_ERR_HIP 4               /* a HIP runtime call or kernel launch failed */
+#define TT_ERR_STATIC_LIMIT 5      /* tt_adaln_backward_static: the shape needs more than TT_STATIC_WORKSPACE_BYTES */
 
 #define TT_MAX_COLS 32768
 
@@ -93,6 +95,23 @@ TT_API int tt_adaln_backward(void* dx, float* dscale, float* dshift,
                       int64_t rows, int64_t cols, int64_t rows_per_batch,
                       float eps, void* stream);
 TT_API size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch);
+
+/* tt_adaln_backward for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without the
+ * workspace, same kernels, same results bit for bit.  No counterpart in the reference.  The
+ * partial column sums live in a device array inside the library, TT_STATIC_WORKSPACE_BYTES
+ * (16 MiB) per GPU, held from the first call on that GPU until the process ends; the call
+ * performs no hipMalloc / hipFree.  A shape whose launch plan needs more (what
+ * tt_adaln_backward_workspace_bytes() returns; 10.2 MB at rows 75600, cols 5120) is refused
+ * with TT_ERR_STATIC_LIMIT.  All calls on one GPU share the array: two calls that overlap in
+ * time on the same GPU (different streams or host threads) race and give wrong dscale / dshift;
+ * calls that follow each other on one stream are safe (nothing in the array has to start at zero).
+ */
+#define TT_STATIC_WORKSPACE_BYTES (16u << 20)
+TT_API int tt_adaln_backward_static(void* dx, float* dscale, float* dshift,
+                             const void* dy, const void* x, const void* scale,
+                             int64_t rows, int64_t cols, int64_t rows_per_batch,
+                             float eps, void* stream);
 
 /* ------------------------------------------------------------------ fused RMSNorm
  * y = x * rsqrt(mean(x^2) + eps) * weight

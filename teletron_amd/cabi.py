@@ -19,6 +19,8 @@ TT_ERR_INVALID_ARGUMENT = 1
 TT_ERR_UNSUPPORTED = 2
 TT_ERR_WORKSPACE = 3
 TT_ERR_HIP = 4
+TT_ERR_STATIC_LIMIT = 5
+TT_STATIC_WORKSPACE_BYTES = 16 << 20
 
 
 class TeletronOpError(RuntimeError):
@@ -39,6 +41,8 @@ PROTOTYPES = {
                                  c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_adaln_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_size_t, c_int64, c_int64, c_int64, c_float, c_void_p]),
+    "tt_adaln_backward_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_adaln_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "tt_rmsnorm_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_int64, c_float, c_void_p]),

@@ -63,6 +63,31 @@ int resident_wgs_per_cu(const KernelInfo& k, int* out) {
   return TT_OK;
 }
 
+// Backward workspace of tt_adaln_backward_static: a file-scope device array, so that the entry
+// point never allocates.  Every device the library runs on holds its own copy at its own address;
+// the host-side name below is only a handle for hipGetSymbolAddress, never a kernel argument.
+static __device__ __align__(256) unsigned char scratch[TT_STATIC_WORKSPACE_BYTES];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  static std::mutex mu;
+  static void* addr[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e);
+  if (dev < 0 || dev >= 64) return TT_ERR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e);
+    if (!p) return TT_ERR_HIP;
+    addr[dev] = p;
+  }
+  *out = addr[dev];
+  return TT_OK;
+}
+
 std::atomic<int> g_wgs_per_cu_override{0};
 std::atomic<int> g_grid_override{0};
 
@@ -405,6 +430,7 @@ const char* tt_error_string(int code) {
     case TT_ERR_UNSUPPORTED: return "unsupported shape or alignment";
     case TT_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case TT_ERR_HIP: return "HIP runtime error (see tt_last_hip_error)";
+    case TT_ERR_STATIC_LIMIT: return "shape needs more than TT_STATIC_WORKSPACE_BYTES of scratch: use the entry point that takes a workspace";
     default: return "unknown error code";
   }
 }
@@ -467,6 +493,18 @@ int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, co
                              rows, cols, rows_per_batch, eps, stream);
   if (rc != TT_OK) return rc;
   return reduce(dscale, dshift, workspace, (int)(rows / rows_per_batch), n_partials, 2, cols, false, stream);
+}
+
+int tt_adaln_backward_static(void* dx, float* dscale, float* dshift, const void* dy, const void* x,
+                             const void* scale, int64_t rows, int64_t cols, int64_t rows_per_batch, float eps,
+                             void* stream) {
+  if (rows == 0) return TT_OK;
+  void* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc != TT_OK) return rc;
+  rc = tt_adaln_backward(dx, dscale, dshift, dy, x, scale, ws, TT_STATIC_WORKSPACE_BYTES,
+                         rows, cols, rows_per_batch, eps, stream);
+  return rc == TT_ERR_WORKSPACE ? TT_ERR_STATIC_LIMIT : rc;
 }
 
 int tt_rmsnorm_backward(void* dx, float* dweight, const void* dy, const void* x, const void* weight,

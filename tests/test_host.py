@@ -35,8 +35,8 @@ def test_library_exports_every_declared_symbol(lib):
 def test_version_and_error_strings(lib):
     assert lib.tt_version() >= 100
     from teletron_amd import cabi
-    texts = {lib.tt_error_string(c) for c in range(0, 6)}
-    assert len(texts) == 6 and b"ok" in texts
+    texts = {lib.tt_error_string(c) for c in range(0, 7)}
+    assert len(texts) == 7 and b"ok" in texts
     assert lib.tt_last_hip_error() == 0
     e = cabi.TeletronOpError("f", 2, "unsupported")
     assert e.code == 2 and "f failed" in str(e)

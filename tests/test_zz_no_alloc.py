@@ -1,0 +1,63 @@
+"""The entry point that allocates nothing (tt_adaln_backward_static) against tt_adaln_backward,
+through the C ABI: same kernels and plan, so the results must agree bit for bit.  Two calls in a
+row share the library's device array; the second is smaller and must not see the first's sums."""
+import pytest
+import torch
+
+from teletron_amd import cabi
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(rows, cols, n_batches, seed):
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g).bfloat16().to(dev)
+    dy = torch.randn(rows, cols, generator=g).bfloat16().to(dev)
+    scale = (0.1 * torch.randn(n_batches, cols, generator=g)).bfloat16().to(dev)
+    rpb = rows // n_batches
+    st = torch.cuda.current_stream().cuda_stream
+    lib = cabi.load()
+    need = lib.tt_adaln_backward_workspace_bytes(rows, cols, rpb)
+    assert need <= cabi.TT_STATIC_WORKSPACE_BYTES
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    ref = [torch.empty_like(x), torch.empty(n_batches, cols, device=dev), torch.empty(n_batches, cols, device=dev)]
+    got = [torch.full_like(x, float("nan")), torch.full((n_batches, cols), float("nan"), device=dev),
+           torch.full((n_batches, cols), float("nan"), device=dev)]
+    cabi.call("tt_adaln_backward", ref[0].data_ptr(), ref[1].data_ptr(), ref[2].data_ptr(), dy.data_ptr(),
+              x.data_ptr(), scale.data_ptr(), ws.data_ptr(), ws.numel(), rows, cols, rpb, 1e-6, st)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    cabi.call("tt_adaln_backward_static", got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(), dy.data_ptr(),
+              x.data_ptr(), scale.data_ptr(), rows, cols, rpb, 1e-6, st)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    for name, a, b in zip(("dx", "dscale", "dshift"), got, ref):
+        assert torch.equal(a, b), f"{name} differs at rows={rows} cols={cols} batches={n_batches}"
+    assert bool(torch.isfinite(got[1]).all()) and bool(torch.isfinite(got[2]).all())
+
+
+def test_static_backward_matches_workspace_backward_twice():
+    print("case: tt_adaln_backward_static rows=6000 cols=5120 batches=2, then rows=1201 cols=1536 batches=1", flush=True)
+    _run(6000, 5120, 2, seed=11)
+    _run(1201, 1536, 1, seed=12)     # smaller input, same device array
+    _run(77, 1000, 1, seed=13)       # ragged width (masked kernel variant)
+
+
+def test_static_backward_limit_and_noop():
+    lib = cabi.load()
+    dev = "cuda:0"
+    # zero rows: nothing to do, no pointer is looked at
+    assert lib.tt_adaln_backward_static(None, None, None, None, None, None, 0, 512, 1, 1e-6, None) == cabi.TT_OK
+    # a shape whose plan needs more than the array holds is refused before any launch
+    rows, cols = 40000, 16384
+    assert lib.tt_adaln_backward_workspace_bytes(rows, cols, rows) > cabi.TT_STATIC_WORKSPACE_BYTES
+    x = torch.zeros(rows, cols, dtype=torch.bfloat16, device=dev)
+    dx = torch.empty_like(x)
+    p = torch.zeros(cols, dtype=torch.bfloat16, device=dev)
+    g0 = torch.empty(cols, device=dev)
+    g1 = torch.empty(cols, device=dev)
+    rc = lib.tt_adaln_backward_static(dx.data_ptr(), g0.data_ptr(), g1.data_ptr(), x.data_ptr(), x.data_ptr(),
+                                      p.data_ptr(), rows, cols, rows, 1e-6, None)
+    assert rc == cabi.TT_ERR_STATIC_LIMIT
+    assert b"TT_STATIC_WORKSPACE_BYTES" in lib.tt_error_string(rc)
