@@ -250,12 +250,17 @@ TT_API int tt_residual_norm_backward(void* dx, void* dr, float* dscale, float* d
 TT_API size_t tt_residual_norm_backward_workspace_bytes(int64_t rows, int64_t cols, int64_t rows_per_batch, int gated);
 
 /* ------------------------------------------------------------------ bare streaming probe
- * Measurement aid without a counterpart in the reference: out[i] = a[i] (b == NULL) or
- * a[i] ^ b[i] over `bytes` bytes, with the load/store policy of the kernels above, one
- * workgroup per compute unit and no arithmetic.  A benchmark runs it on the same buffers to report
- * what plain one-read-one-write and two-reads-one-write traffic reaches on the machine at hand,
- * next to the published HBM peak.  bytes % 16 == 0 and 16-byte aligned pointers
- * (TT_ERR_UNSUPPORTED otherwise); bytes == 0 is a no-op. */
+ * Measurement aid without a counterpart in the reference.  Over `bytes` bytes, with the
+ * load/store policy of the kernels above, one workgroup per compute unit and no arithmetic:
+ *   out, a        out[i] = a[i]                       (one read, one write)
+ *   out, a, b     out[i] = a[i] ^ b[i]                (two reads, one write)
+ *   a only        a is read and dropped               (out == NULL: reads on their own)
+ *   out only      every 16-byte pack of out receives its own index (low 32 bits) in each of its
+ *                 four words                          (a == NULL: writes on their own)
+ * A benchmark runs it on the same buffers to report what each traffic mix reaches on the
+ * machine at hand, next to the published HBM peak.  bytes % 16 == 0 and 16-byte aligned pointers
+ * (TT_ERR_UNSUPPORTED otherwise); bytes == 0 is a no-op; out == a == NULL, or b without both
+ * out and a, is TT_ERR_INVALID_ARGUMENT. */
 TT_API int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void* stream);
 
 /* ------------------------------------------------------------------ reference-compatible contract

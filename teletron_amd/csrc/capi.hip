@@ -664,7 +664,7 @@ int tt_residual_norm_backward(void* dx, void* dr, float* dscale, float* dshift, 
 // ---------------------------------------------------------------- bare streaming probe
 int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void* stream) {
   if (bytes == 0) return TT_OK;
-  if (!out || !a) return TT_ERR_INVALID_ARGUMENT;
+  if ((!out && !a) || (b && (!out || !a))) return TT_ERR_INVALID_ARGUMENT;
   if (bytes % 16 != 0 || !aligned16(out) || !aligned16(a) || !aligned16(b)) return TT_ERR_UNSUPPORTED;
   int cus = 0;
   const int rc = current_device_cus(&cus);
@@ -673,8 +673,11 @@ int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void*
   const size_t want = (n + kProbeThreads - 1) / kProbeThreads;
   const dim3 grid((unsigned)(want < (size_t)cus ? want : (size_t)cus));   // one workgroup per CU
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (b) hipLaunchKernelGGL((stream_probe<true, 1>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
-  else   hipLaunchKernelGGL((stream_probe<false, 2>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  // packs per lane in flight: what streams fastest for each mix with one 512-thread workgroup per CU
+  if (!out)    hipLaunchKernelGGL((stream_probe<kProbeRead, 4>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  else if (!a) hipLaunchKernelGGL((stream_probe<kProbeWrite, 4>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  else if (b)  hipLaunchKernelGGL((stream_probe<kProbeXor, 1>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  else         hipLaunchKernelGGL((stream_probe<kProbeCopy, 2>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? TT_OK : hip_fail(e);
 }

@@ -1,6 +1,7 @@
 // Bare streaming kernels with the load/store policy of the normalisation kernels and no
-// arithmetic: what one-read-one-write and two-reads-one-write traffic reaches on the machine at
-// hand.  Measurement aid for benchmarks; the product kernels do not use them.
+// arithmetic: what one-read-one-write and two-reads-one-write traffic, and reads or writes on
+// their own, reach on the machine at hand.  Measurement aid for benchmarks; the product kernels
+// do not use them.
 #pragma once
 #include "common.hpp"
 
@@ -8,9 +9,14 @@ namespace tt {
 
 constexpr int kProbeThreads = 512;
 
-// out[i] = a[i] (TWO == false) or a[i] ^ b[i] (TWO == true) over n 128-bit packs; grid-stride,
-// U packs per lane in flight.
-template <bool TWO, int U>
+enum ProbeMode : int { kProbeCopy = 0, kProbeXor = 1, kProbeRead = 2, kProbeWrite = 3 };
+
+// Over n 128-bit packs, grid-stride, U packs per lane in flight:
+//   kProbeCopy   out[i] = a[i]
+//   kProbeXor    out[i] = a[i] ^ b[i]
+//   kProbeRead   a[i] is loaded and dropped (the empty asm keeps the load and its wait alive)
+//   kProbeWrite  out[i] = the pack's index, low 32 bits, in each of its four words
+template <int MODE, int U>
 __global__ void __launch_bounds__(kProbeThreads) stream_probe(void* __restrict__ out, const void* __restrict__ a,
                                                              const void* __restrict__ b, size_t n) {
   const size_t stride = (size_t)gridDim.x * kProbeThreads;
@@ -19,15 +25,19 @@ __global__ void __launch_bounds__(kProbeThreads) stream_probe(void* __restrict__
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t j = i + u * stride;
+      const unsigned w = (unsigned)j;
+      va[u] = u32x4{w, w, w, w};
+      vb[u] = u32x4{0, 0, 0, 0};
       if (j < n) {
-        va[u] = load_stream(a, j * kPack);
-        if (TWO) vb[u] = load_stream(b, j * kPack);
+        if (MODE != kProbeWrite) va[u] = load_stream(a, j * kPack);
+        if (MODE == kProbeXor) vb[u] = load_stream(b, j * kPack);
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t j = i + u * stride;
-      if (j < n) store_stream(out, j * kPack, TWO ? (va[u] ^ vb[u]) : va[u]);
+      if (MODE == kProbeRead) asm volatile("" ::"v"(va[u]));
+      else if (j < n) store_stream(out, j * kPack, va[u] ^ vb[u]);
     }
   }
 }
