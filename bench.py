@@ -33,8 +33,10 @@ HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E peak
 # known size); the counters cannot be read from inside this process, so the measured figures are
 # carried here.  Valid only while the backward kernel writes the stated number of partial sums.
 MEASURED_TRAFFIC_BYTES = {
-    "adaln_wan14b": {"fwd": 1548486725, "bwd": 2332780526, "n_partials": 248},
+    "adaln_wan14b": {"fwd": 1548486725, "bwd": 2332780526, "n_partials": 248,
+                     "source": "profiles/adaln_wan14b_hbm_traffic_pmc.md"},
 }
+CACHE_RESIDENT_BYTES = 64 << 20   # tensors below this size are served from the caches
 METRIC = "fwd+bwd HBM GB/s and % of peak, AdaLN/RMSNorm at Wan-14B shape 75600x5120"
 
 
@@ -48,7 +50,8 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
     ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched,"
                                       "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
-                                      "residual_adaln_wan14b,gated_residual_layernorm_wan14b,rmsnorm_rope_hunyuan_head",
+                                      "residual_adaln_wan14b,gated_residual_layernorm_wan14b,rmsnorm_rope_hunyuan_head,"
+                                      "rmsnorm_small,adaln_odd",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--no-eager-gpu", action="store_true", help="skip timing the eager PyTorch expressions on the GPU")
     ap.add_argument("--block-demo", action="store_true",
@@ -57,6 +60,11 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
                          "that hardware byte counters collected over this run can be scaled against it")
+    ap.add_argument("--no-function-path", action="store_true",
+                    help="skip timing the autograd Functions (the path model code calls) at the workload's shape")
+    ap.add_argument("--ceiling-sweep", action="store_true",
+                    help="run teletron_amd/ceiling_sweep (bare read / write / copy / 2r1w streams under every address "
+                         "layout and store path) and print its table instead of the benchmark line")
     return ap.parse_args()
 
 
@@ -215,19 +223,22 @@ class GpuWorkload:
         torch = self.torch
         nbytes = self.rows * self.cols * 2
 
-        def timed(two):
+        def timed(mix):
             ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters + 3)]
             for i, e in enumerate(ev):
                 s = self.sets[i % len(self.sets)]
+                out = None if mix == "read" else (s["dx"] if mix == "2r1w" else s["y"]).data_ptr()
+                a = None if mix == "write" else s["x"].data_ptr()
+                b = s["dy"].data_ptr() if mix == "2r1w" else None
                 e[0].record()
-                self.cabi.call("tt_stream_probe", (s["dx"] if two else s["y"]).data_ptr(), s["x"].data_ptr(),
-                               s["dy"].data_ptr() if two else None, nbytes, self.stream)
+                self.cabi.call("tt_stream_probe", out, a, b, nbytes, self.stream)
                 e[1].record()
             torch.cuda.synchronize()
             t = statistics.median(e[0].elapsed_time(e[1]) for e in ev[3:]) * 1e-3
-            return (3 if two else 2) * nbytes / t / 1e9
+            return {"read": 1, "write": 1, "copy": 2, "2r1w": 3}[mix] * nbytes / t / 1e9
 
-        return {"copy": timed(False), "two_reads_one_write": timed(True)}
+        return {"copy": timed("copy"), "two_reads_one_write": timed("2r1w"),
+                "read_only": timed("read"), "write_only": timed("write")}
 
     def run(self, steps, warmup):
         """Returns wall seconds per step and per-kernel mean microseconds from HIP events."""
@@ -440,13 +451,55 @@ def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3
             "relative_output_difference": diff, "swapped": counts}
 
 
-def cpu_baseline(w, seconds):
-    """PyTorch-eager fwd + autograd bwd of the same op on the host CPU, bounded row sample."""
+def function_path(w, cabi_ms, iters=10):
+    """The path model code calls: AdaLNModelFunction / RMSNormModelFunction apply + backward on
+    tensors of the workload's shape, parameters as the model passes them ([B, 1, C] modulation,
+    [C] weight), two alternating input sets.  Wall milliseconds per forward+backward and the
+    ratio to the C-ABI step of the same workload."""
+    import torch
+    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction
+    dev, bf = "cuda:0", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(2)
+    rnd = lambda *shape, scale=1.0, offset=0.0: (offset + scale * torch.randn(*shape, generator=g, device=dev)).to(bf)
+    xs = [rnd(*w.shape).requires_grad_(True) for _ in range(2)]
+    dys = [rnd(*w.shape) for _ in range(2)]
+    if w.op == "adaln":
+        scale = rnd(*w.param_shape, scale=0.1).requires_grad_(True)
+        shift = rnd(*w.param_shape, scale=0.1).requires_grad_(True)
+        params = [scale, shift]
+        op = lambda i: AdaLNModelFunction.apply(xs[i], scale, shift, w.eps, w.cols)
+        name = "AdaLNModelFunction"
+    else:
+        weight = rnd(*w.param_shape, scale=0.1, offset=1.0).requires_grad_(True)
+        params = [weight]
+        op = lambda i: RMSNormModelFunction.apply(xs[i], weight, w.eps, w.cols)
+        name = "RMSNormModelFunction"
+
+    def fn(i):
+        for t in [xs[i]] + params:
+            t.grad = None               # no accumulation pass into an existing .grad
+        op(i).backward(dys[i])
+
+    for i in range(4):
+        fn(i & 1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(iters):
+        fn(i & 1)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / iters * 1e3
+    return {"function": name, "ms_per_step": round(ms, 4), "ratio_to_c_abi_step": round(ms / cabi_ms, 4),
+            "note": "apply + backward through torch.autograd, .grad cleared before each step"}
+
+
+def cpu_baseline(w, seconds, full=False):
+    """PyTorch-eager fwd + autograd bwd of the same op on the host CPU; a bounded row sample of
+    the workload, or (full=True) the whole workload."""
     import torch
     from oracle import eager_reference as E
     from teletron_amd.workloads import make_inputs
     threads = torch.get_num_threads()
-    sample_rows = min(w.shape[1], 16384)
+    sample_rows = w.shape[1] if full else min(w.shape[1], 16384)
     t = make_inputs(w, seed=0, rows=sample_rows)
     elements = t["x"].numel()
     if w.op in ("resnorm", "resnorm_gated"):
@@ -472,8 +525,9 @@ def cpu_baseline(w, seconds):
     med = statistics.median(times)
     per_elt = w.algorithmic_bytes("fwd+bwd") / w.elements
     return {"value": round(per_elt * elements / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{w.op} eager bf16 fwd+autograd bwd on x{list(t['x'].shape)} (first {sample_rows} rows of the "
-                      f"workload), median of {len(times)} runs, {med * 1e3:.1f} ms/run, "
+            "sample": f"{w.op} eager bf16 fwd+autograd bwd on x{list(t['x'].shape)} ("
+                      + ("the whole workload" if sample_rows == w.shape[1] else f"first {sample_rows} rows of the workload")
+                      + f"), median of {len(times)} runs, {med * 1e3:.1f} ms/run, "
                       f"{t['x'].numel() // w.cols / med:.3e} rows/s, {per_elt:.0f} B/element"}
 
 
@@ -508,6 +562,13 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HIP kernels have no CPU fallback.", file=sys.stderr)
         return 2
+    if args.ceiling_sweep:
+        import subprocess
+        exe = os.path.join(REPO_ROOT, "teletron_amd", "ceiling_sweep")
+        if not os.path.exists(exe):
+            print(f"{exe} is missing: run `python -m teletron_amd.build` first.", file=sys.stderr)
+            return 2
+        return subprocess.run([exe]).returncode
     w = WORKLOADS[args.workload]
     r = measure(w, args.steps, args.warmup, ceiling=True)
     mt = MEASURED_TRAFFIC_BYTES.get(w.name)
@@ -525,6 +586,8 @@ def main():
                        "reduce_partials": round(r["reduce_us"], 2)},
         "roofline": {"bound": "hbm", "achieved": round(r["bwd_gbps"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(r["bwd_gbps"] / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "traffic_source": (mt["source"] + " (rocprofv3 --pmc run of this command; not re-measured here)")
+                     if traffic else None,
                      "kernel": "norm_bwd_wide (backward streaming kernel)",
                      "algorithmic_bytes_per_launch": w.algorithmic_bytes("bwd"),
                      "forward_kernel": {"achieved": round(r["fwd_gbps"], 1),
@@ -536,6 +599,7 @@ def main():
     c = r["ceiling"]
     out["stream_ceiling"] = {
         "unit": "GB/s", "copy": round(c["copy"], 1), "two_reads_one_write": round(c["two_reads_one_write"], 1),
+        "read_only": round(c["read_only"], 1), "write_only": round(c["write_only"], 1),
         "forward_frac_of_copy": round(r["fwd_gbps"] / c["copy"], 4),
         "backward_frac_of_two_reads_one_write": round(r["bwd_gbps"] / c["two_reads_one_write"], 4),
         "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers"}
@@ -551,6 +615,9 @@ def main():
         also[name] = {"value": round(ra["gbps"], 1), "unit": "GB/s", "pct_of_peak": round(100 * ra["gbps"] / HBM_PEAK_GBPS, 2),
                       "ms_per_step": round(ra["ms_per_step"], 4), "forward_us": round(ra["fwd_us"], 2),
                       "backward_streaming_us": round(ra["bwd_us"], 2), "reduce_partials_us": round(ra["reduce_us"], 2)}
+        if wa.elements * 2 < CACHE_RESIDENT_BYTES:
+            # every tensor fits the 256 MB Infinity Cache: reported, not an HBM figure
+            also[name]["cache_resident"] = True
         if not args.no_eager_gpu:
             ms = eager_gpu(wa, iters=3)
             if ms:
@@ -567,8 +634,14 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         out["calibration_copy_bytes"] = src.numel() * 2
+    if not args.no_function_path and w.op in ("adaln", "rmsnorm") and w.contract == "native":
+        out["function_path"] = function_path(w, r["ms_per_step"])
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+        small = WORKLOADS["rmsnorm_small"]
+        if small.name != w.name:
+            # the reference's own CPU-runnable configuration, at full size
+            out["cpu_baseline_also"] = {small.name: cpu_baseline(small, min(args.cpu_seconds, 6.0), full=True)}
     print(json.dumps(out))
     return 0
 

@@ -67,10 +67,25 @@ def build_library(force: bool = True, defines=(), jobs: int = 8, verbose: bool =
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
-    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", f"-Wl,-soname,{LIB_PATH.name}", "-o", str(LIB_PATH),
+          *map(str, objs)])
     if verbose:
         print("[teletron_amd.build] linked", LIB_PATH, flush=True)
     return LIB_PATH
+
+
+SWEEP_PATH = PKG_DIR / "ceiling_sweep"
+
+
+def build_ceiling_sweep(verbose: bool = True) -> Path:
+    """Compile the stand-alone stream-ceiling measurement program (csrc/ceiling_sweep.hip), which
+    ``bench.py --ceiling-sweep`` runs.  It does not link against the library."""
+    if verbose:
+        print("[teletron_amd.build] hipcc ceiling_sweep.hip", flush=True)
+    _run([hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-o", str(SWEEP_PATH),
+          str(CSRC / "ceiling_sweep.hip")])
+    return SWEEP_PATH
 
 
 TORCH_EXT_MODULES = ["fused_adaln", "fused_rmsnorm"]
@@ -107,7 +122,7 @@ def build_torch_extensions(force: bool = True, verbose: bool = True):
                f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H",
                f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-deprecated-declarations", *incs, str(src), "-o", str(out),
                f"-L{torch_lib}", "-L/opt/rocm/lib", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip",
-               "-ltorch_hip", "-lamdhip64", str(LIB_PATH),
+               "-ltorch_hip", "-lamdhip64", f"-L{PKG_DIR}", f"-l:{LIB_PATH.name}",
                "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}", "-Wl,-rpath,/opt/rocm/lib"]
         if verbose:
             print("[teletron_amd.build] g++", src.name, flush=True)
@@ -128,6 +143,7 @@ def main(argv=None) -> int:
     build_library(force=args.force or bool(args.define), defines=args.define, jobs=args.jobs)
     if not args.no_torch_ext:
         build_torch_extensions(force=args.force)
+    build_ceiling_sweep()
     return 0
 
 

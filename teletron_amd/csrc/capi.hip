@@ -670,14 +670,16 @@ int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void*
   const int rc = current_device_cus(&cus);
   if (rc != TT_OK) return rc;
   const size_t n = bytes / 16;
-  const size_t want = (n + kProbeThreads - 1) / kProbeThreads;
-  const dim3 grid((unsigned)(want < (size_t)cus ? want : (size_t)cus));   // one workgroup per CU
+  // One workgroup per CU; threads and packs per lane in flight are what streamed fastest for each
+  // mix on MI355X (reads want many requests in flight, writes few: 4 waves with one store each).
+  const int threads = !a ? 256 : kProbeMaxThreads;
+  const size_t want = (n + threads - 1) / threads;
+  const dim3 grid((unsigned)(want < (size_t)cus ? want : (size_t)cus));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // packs per lane in flight: what streams fastest for each mix with one 512-thread workgroup per CU
-  if (!out)    hipLaunchKernelGGL((stream_probe<kProbeRead, 4>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
-  else if (!a) hipLaunchKernelGGL((stream_probe<kProbeWrite, 4>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
-  else if (b)  hipLaunchKernelGGL((stream_probe<kProbeXor, 1>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
-  else         hipLaunchKernelGGL((stream_probe<kProbeCopy, 2>), grid, dim3(kProbeThreads), 0, s, out, a, b, n);
+  if (!out)    hipLaunchKernelGGL((stream_probe<kProbeRead, 4>), grid, dim3(threads), 0, s, out, a, b, n);
+  else if (!a) hipLaunchKernelGGL((stream_probe<kProbeWrite, 1>), grid, dim3(threads), 0, s, out, a, b, n);
+  else if (b)  hipLaunchKernelGGL((stream_probe<kProbeXor, 1>), grid, dim3(threads), 0, s, out, a, b, n);
+  else         hipLaunchKernelGGL((stream_probe<kProbeCopy, 2>), grid, dim3(threads), 0, s, out, a, b, n);
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? TT_OK : hip_fail(e);
 }

@@ -501,7 +501,9 @@ __global__ __launch_bounds__(64 * W * Q) void norm_bwd_wide(const BwdArgs a) {
 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float rstd = rsqrtf(red_v[r * NV + 0] * a.inv_cols + a.eps);
+      // rows past the end of the batch (zero-filled) must stay out of the column sums even when
+      // eps == 0 would turn their rstd into inf
+      const float rstd = rv[r] ? rsqrtf(red_v[r * NV + 0] * a.inv_cols + a.eps) : 0.f;
       // dx = rstd*g - rstd*mean(g) - x_hat * rstd*mean(g*x_hat),  mean(g*x_hat) = rstd * sum(g*d) / C
       const float k2 = -(rstd * rstd) * (red_v[r * NV + 1] * a.inv_cols);
       const float k1 = ADALN ? -rstd * (red_v[r * NV + 2] * a.inv_cols) : 0.f;
@@ -808,7 +810,7 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       sv = group_allsum<L>(sv);
       sh_ = group_allsum<L>(sh_);
       if constexpr (ADALN) sg = group_allsum<L>(sg);
-      const float rstd = rsqrtf(sv * a.inv_cols + a.eps);
+      const float rstd = rv[r] ? rsqrtf(sv * a.inv_cols + a.eps) : 0.f;   // padding rows: see the wide kernel
       const float k2 = -(rstd * rstd) * (sh_ * a.inv_cols);
       const float k1 = ADALN ? -rstd * (sg * a.inv_cols) : 0.f;
       float o[8];

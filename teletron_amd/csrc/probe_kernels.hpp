@@ -7,20 +7,21 @@
 
 namespace tt {
 
-constexpr int kProbeThreads = 512;
+constexpr int kProbeMaxThreads = 512;
 
 enum ProbeMode : int { kProbeCopy = 0, kProbeXor = 1, kProbeRead = 2, kProbeWrite = 3 };
 
-// Over n 128-bit packs, grid-stride, U packs per lane in flight:
+// Over n 128-bit packs, grid-stride, U packs per lane in flight, any workgroup size up to
+// kProbeMaxThreads:
 //   kProbeCopy   out[i] = a[i]
 //   kProbeXor    out[i] = a[i] ^ b[i]
 //   kProbeRead   a[i] is loaded and dropped (the empty asm keeps the load and its wait alive)
 //   kProbeWrite  out[i] = the pack's index, low 32 bits, in each of its four words
 template <int MODE, int U>
-__global__ void __launch_bounds__(kProbeThreads) stream_probe(void* __restrict__ out, const void* __restrict__ a,
+__global__ void __launch_bounds__(kProbeMaxThreads) stream_probe(void* __restrict__ out, const void* __restrict__ a,
                                                              const void* __restrict__ b, size_t n) {
-  const size_t stride = (size_t)gridDim.x * kProbeThreads;
-  for (size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x; i < n; i += U * stride) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += U * stride) {
     u32x4 va[U], vb[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {

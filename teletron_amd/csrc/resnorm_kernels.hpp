@@ -368,7 +368,7 @@ __global__ __launch_bounds__(64 * W * Q) void resnorm_bwd_wide(const ResBwdArgs 
 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float rstd = rsqrtf(red_v[r * NV + 0] * a.inv_cols + a.eps);
+      const float rstd = rv[r] ? rsqrtf(red_v[r * NV + 0] * a.inv_cols + a.eps) : 0.f;   // zero-filled padding rows stay out of the column sums
       const float k2 = -(rstd * rstd) * (red_v[r * NV + 1] * a.inv_cols);
       const float k1 = -rstd * (red_v[r * NV + 2] * a.inv_cols);
       const int64_t row = b * S + row0 + r;

@@ -74,13 +74,29 @@ def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int,
     return rows, nb, (rows // nb if nb else rows)
 
 
+_WORKSPACES = {}   # (device index, stream handle) -> uint8 tensor, grown on demand
+
+
 def _workspace(lib_bytes: int, rows: int, *tensors: torch.Tensor) -> torch.Tensor:
-    """Backward workspace; tensors that are not 16-byte aligned take the element-wise kernels,
-    which keep two floats of statistics per row there."""
+    """Backward workspace (partial column sums), kept per device and stream and reused from call to
+    call: launches on one stream run in order, so consecutive backward calls never overlap in it.
+    Tensors that are not 16-byte aligned take the element-wise kernels, which keep two floats of
+    statistics per row there."""
     need = lib_bytes
     if any(t.data_ptr() % 16 for t in tensors):
         need = max(need, rows * 8)
-    return torch.empty(max(need, 16), dtype=torch.uint8, device=tensors[0].device)
+    need = max(need, 16)
+    dev = tensors[0].device
+    if torch.cuda.is_current_stream_capturing():
+        # a captured graph keeps the pointers it recorded: give it memory of its own (from the
+        # capture's private pool), never the shared buffer
+        return torch.empty(need, dtype=torch.uint8, device=dev)
+    key = (dev.index, _stream(tensors[0]))
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        _WORKSPACES[key] = ws
+    return ws
 
 
 def _stream(t: torch.Tensor) -> int:

@@ -35,6 +35,7 @@ def assert_bf16_close(got, ref, what):
     ref = ref.double().reshape(-1)
     err = (got - ref).abs()
     bound = 1e-2 + 8e-3 * ref.abs()
+    assert bool(torch.isfinite(got).all()), f"{what}: non-finite values"
     bad = err > bound
     assert not bad.any(), f"{what}: {int(bad.sum())} of {ref.numel()} outside tolerance, worst excess {float((err - bound).max()):.3e}"
 
@@ -44,6 +45,7 @@ def assert_grad_close(got, ref, rows_reduced, what):
     ref = ref.double().reshape(-1)
     err = (got - ref).abs()
     bound = 1e-3 * ref.abs() + 1e-4 * math.sqrt(rows_reduced)
+    assert bool(torch.isfinite(got).all()), f"{what}: non-finite values"
     bad = err > bound
     assert not bad.any(), f"{what}: {int(bad.sum())} of {ref.numel()} outside tolerance, worst err {float(err.max()):.3e}"
 
@@ -143,6 +145,22 @@ def test_rmsnorm_shapes(cols, rows):
     gamma = rand_bf16(cols, seed=seed + 1, scale=0.1, offset=1.0)
     dy = rand_bf16(rows, cols, seed=seed + 2)
     check_rmsnorm(x, gamma, dy, 1e-6, f"rmsnorm[{rows},{cols}]")
+
+
+@pytest.mark.parametrize("cols", [128, 1536, 5120])
+def test_eps_zero_with_ragged_row_tail(cols):
+    """eps = 0 and a row count that leaves part of the last tile empty: the zero-filled padding rows
+    must not reach the column sums (their rstd would be inf), so the parameter gradients stay finite
+    and equal to the oracle's."""
+    for nb, rpb in [(1, 67), (2, 29)]:
+        seed = cols + rpb
+        x = rand_bf16(nb, rpb, cols, seed=seed, offset=0.5)
+        scale = rand_bf16(nb, 1, cols, seed=seed + 1, scale=0.1)
+        shift = rand_bf16(nb, 1, cols, seed=seed + 2, scale=0.1)
+        dy = rand_bf16(nb, rpb, cols, seed=seed + 3)
+        check_adaln(x, scale, shift, dy, 0.0, nb, f"adaln eps=0 [{nb},{rpb},{cols}]")
+        check_rmsnorm(x.reshape(-1, cols), rand_bf16(cols, seed=seed + 4, scale=0.1, offset=1.0),
+                      dy.reshape(-1, cols), 0.0, f"rmsnorm eps=0 [{nb * rpb},{cols}]")
 
 
 # ------------------------------------------------------------------ element-wise path: odd widths, misaligned tensors

@@ -179,3 +179,19 @@ def test_swap_in_leaves_context_parallel_callables_alone_with_several_ranks(monk
     assert isinstance(many.norm1, nn.LayerNorm)
     assert not hasattr(many.modulate_with_cp_grad_reduce, "__wrapped__")
     assert "forward" not in many.__dict__
+
+
+def test_glue_modules_find_the_library_by_name_not_by_build_path():
+    """The pybind modules must record libteletron_op.so by its soname (found through their
+    $ORIGIN rpath), so that the package still loads after it has been copied elsewhere."""
+    import subprocess
+    from teletron_amd import build as tb
+    for name in tb.TORCH_EXT_MODULES:
+        path = tb.torch_ext_path(name)
+        if not path.exists():
+            pytest.skip(f"{path.name} not built")
+        out = subprocess.run(["readelf", "-d", str(path)], capture_output=True, text=True, check=True).stdout
+        needed = re.findall(r"\(NEEDED\).*\[(.*)\]", out)
+        assert "libteletron_op.so" in needed, needed
+        assert not [n for n in needed if "/" in n], needed
+        assert "$ORIGIN" in out
