@@ -32,6 +32,14 @@ ships no code that performs the swap.  This module does it by patching *instance
   ``norm_k`` and the ``rope_apply`` after them as one kernel per tensor
   (:func:`fused_self_attention_forward`).
 
+* HunyuanVideo (``teletron/models/hunyuan/model.py``): ``norm2`` / ``norm2_context`` of
+  ``HunyuanVideoTransformerBlock`` with the inline modulation after them (``:615-623,660-669``) go
+  the token way as well; the ``gate(self, x, gate, residual)`` *methods* of both block classes
+  (``:538-539,627-628``) are shadowed by the fused gated residual add; with ``blocks=True`` every
+  attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
+  :class:`FusedHunyuanAttnProcessor`, which runs ``norm_q`` / ``norm_k`` and the rotary embedding
+  after them as one kernel per tensor (text tokens appended to the latent ones take no rotation).
+
 Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` / ``gate_with_cp_grad_reduce``
 all-reduce their parameter gradients over the context-parallel group
 (``core/context_parallel/layers.py:31-36,46-53``); with a group of size 1 that is the identity,
@@ -49,10 +57,16 @@ import torch.nn as nn
 
 from . import ops
 from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, RMSNormRopeFunction,
-                         adaln_modulate, residual_adaln, residual_layer_norm)
+                         RMSNormRopeHeadsFunction, adaln_modulate, residual_adaln, residual_layer_norm,
+                         rope_table_from_cos_sin)
 
-ADALN_NORM_ATTRS = ("norm1", "norm2", "norm")
-ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle")
+ADALN_NORM_ATTRS = ("norm1", "norm2", "norm", "norm2_context")
+ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle",
+                       "HunyuanVideoTransformerBlock")     # hunyuan/model.py:615-623: norm2, norm2_context, inline form
+# classes whose ``gate(self, x, gate, residual)`` is a method (hunyuan/model.py:538-539,627-628); context
+# parallelism replaces it by attribute assignment (hunyuan/parallel_model.py:239-244)
+GATE_METHOD_OWNERS = ("HunyuanVideoSingleTransformerBlock", "HunyuanVideoTransformerBlock")
+HUNYUAN_PROCESSOR = "HunyuanVideoAttnProcessor2_0"         # hunyuan/model.py:64-170 (the one-GPU processor)
 MODULATE_ATTRS = ("modulate", "modulate_with_cp_grad_reduce")
 GATE_ATTRS = ("gate_with_cp_grad_reduce",)                   # context_parallel/layers.py:20-21, parallel_wan_model.py:26,35
 CP_ATTRS = ("modulate_with_cp_grad_reduce", "gate_with_cp_grad_reduce")
@@ -83,8 +97,11 @@ class DeferredNorm:
     def __add__(self, shift):
         if self.one_plus_scale is None or not isinstance(shift, torch.Tensor):
             raise TypeError("DeferredNorm supports exactly `norm(x) * (1 + scale) + shift`")
-        # (1 + scale) was rounded to the activation dtype by the caller; subtracting 1 is exact
-        # there, so the kernel multiplies by the very factor the eager expression would use.
+        # (1 + scale) was rounded to the activation dtype by the caller.  Subtracting 1 again is
+        # exact while 0.5 <= 1 + scale <= 2 (Sterbenz); outside that range it can lose the last
+        # bit of the rounded factor, far below the bf16 resolution of the output.
+        if not _same_dtype(self.x, shift, self.one_plus_scale):   # wider modulation: eager, which promotes
+            return self.materialize() * self.one_plus_scale + shift
         return modulate_token(self, shift, self.one_plus_scale - 1)
 
     __radd__ = __add__
@@ -101,6 +118,8 @@ class DeferredNorm:
 
 def modulate_token(token: DeferredNorm, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     x = token.x
+    if not _same_dtype(x, shift, scale):      # wider modulation: the eager expression, which promotes
+        return token.materialize() * (1 + scale) + shift
     return AdaLNModelFunction.apply(x, scale, shift, token.eps, x.shape[-1])
 
 
@@ -120,8 +139,7 @@ def fused_gate(original: Callable) -> Callable:
     """Wrap a ``gate(x, gate, residual)`` callable: bf16 GPU tensors take the fused kernel."""
 
     def gate(x, gate, residual):
-        if (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16
-                and residual.dtype == torch.bfloat16 and x.shape == residual.shape):
+        if _gate_fusable(x, gate, residual):
             return GateResidualFunction.apply(x, gate, residual)
         return original(x, gate, residual)
 
@@ -158,18 +176,32 @@ class DeferredLayerNorm(nn.Module):
 
 
 def _is_rmsnorm(m: nn.Module) -> bool:
+    """Wan's RMSNorm (wan_model.py:113-124) or the diffusers one HunyuanVideo uses for qk_norm:
+    a 1-D ``weight``, an ``eps`` and no bias."""
     return (type(m).__name__ == "RMSNorm" and isinstance(getattr(m, "weight", None), nn.Parameter)
-            and m.weight.dim() == 1 and hasattr(m, "eps"))
+            and m.weight.dim() == 1 and hasattr(m, "eps") and getattr(m, "bias", None) is None)
+
+
+def _same_dtype(x: torch.Tensor, *params) -> bool:
+    """The fused kernels compute with bf16 parameters and return bf16.  Eager code promotes to the
+    parameter's dtype when that is wider (fp32 master weights under autocast), so only inputs whose
+    parameters are bf16 as well take the fused path; everything else stays on the original one."""
+    return all(p is None or p.dtype == x.dtype for p in params)
 
 
 def _fused_rmsnorm_forward(self, x: torch.Tensor) -> torch.Tensor:
-    if x.is_cuda and x.dtype == torch.bfloat16:
+    if x.is_cuda and x.dtype == torch.bfloat16 and _same_dtype(x, self.weight):
         return RMSNormModelFunction.apply(x, self.weight, self.eps, x.shape[-1])
     return type(self).forward(self, x)
 
 
+def _gate_fusable(x, gate, residual) -> bool:
+    return (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16 and isinstance(residual, torch.Tensor)
+            and residual.dtype == torch.bfloat16 and x.shape == residual.shape and _same_dtype(x, gate))
+
+
 def _fused_gate_forward(self, x, gate, residual):
-    if x.is_cuda and x.dtype == torch.bfloat16 and residual.dtype == torch.bfloat16 and x.shape == residual.shape:
+    if _gate_fusable(x, gate, residual):
         return GateResidualFunction.apply(x, gate, residual)
     return type(self).forward(self, x, gate, residual)
 
@@ -185,7 +217,7 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
     """``DiTBlock.forward`` (``wan_model.py:231-244``; ``parallel_wan_model.py:18-37`` is the same
     sequence) with the norm + modulate pairs and both residual updates on the fused kernels.  The
     sub-modules (``self_attn``, ``cross_attn``, ``ffn``) and all parameters are used as they are."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16):
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and _same_dtype(x, t_mod, self.norm3.weight, self.norm3.bias)):
         return type(self).forward(self, x, context, t_mod, freqs)
     shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
         self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
@@ -205,12 +237,79 @@ def fused_self_attention_forward(self, x, freqs):
     q, k = self.q(x), self.k(x)
     head_dim = q.shape[-1] // self.num_heads
     if not (q.is_cuda and q.dtype == torch.bfloat16 and q.shape[-1] > 256 and head_dim % 8 == 0 and head_dim <= 256
-            and q.dim() >= 2 and freqs.shape[0] == q.shape[-2]):
+            and q.dim() >= 2 and freqs.shape[0] == q.shape[-2] and _same_dtype(q, self.norm_q.weight, self.norm_k.weight)):
         return type(self).forward(self, x, freqs)
     table = ops._check_freqs(freqs.detach(), q, head_dim)          # converted once, shared by q and k
     q = RMSNormRopeFunction.apply(q, self.norm_q.weight, table, self.norm_q.eps, self.num_heads)
     k = RMSNormRopeFunction.apply(k, self.norm_k.weight, table, self.norm_k.eps, self.num_heads)
     return self.o(self.attn(q, k, self.v(x)))
+
+
+class FusedHunyuanAttnProcessor:
+    """``HunyuanVideoAttnProcessor2_0.__call__`` (``teletron/models/hunyuan/model.py:71-170``) with
+    the per-head ``attn.norm_q`` / ``attn.norm_k`` and the ``apply_rotary_emb`` that follows them
+    (``:92-121``) as one kernel per tensor.  In the single-stream blocks the text tokens are
+    appended to the latent ones before the projections and take no rotation (``:101-119``): their
+    rows of the (cos, sin) table are (1, 0).  Projections, the text-stream projections and norms,
+    the attention itself and the output projections are the module's own.  Whatever the fused
+    kernel does not cover (no rotary table, no RMSNorm on q / k, other dtypes) goes to the original
+    processor unchanged."""
+
+    def __init__(self, original):
+        self.original = original
+
+    @staticmethod
+    def _fusable(attn, hidden_states, image_rotary_emb) -> bool:
+        if not (isinstance(image_rotary_emb, (tuple, list)) and len(image_rotary_emb) == 2):
+            return False
+        nq, nk = getattr(attn, "norm_q", None), getattr(attn, "norm_k", None)
+        if not (_is_rmsnorm(nq) and _is_rmsnorm(nk)):
+            return False
+        cos, sin = image_rotary_emb
+        d = nq.weight.shape[0]
+        return (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 3
+                and _same_dtype(hidden_states, nq.weight, nk.weight) and d % 8 == 0 and d <= 256
+                and nk.weight.shape[0] == d and cos.dim() == 2 and cos.shape == sin.shape
+                and cos.shape == (hidden_states.shape[1], d))
+
+    def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None):
+        if not self._fusable(attn, hidden_states, image_rotary_emb):
+            return self.original(attn, hidden_states, encoder_hidden_states, attention_mask, image_rotary_emb)
+        import torch.nn.functional as F
+        single_stream = attn.add_q_proj is None and encoder_hidden_states is not None
+        n_text = encoder_hidden_states.shape[1] if single_stream else 0
+        if single_stream:
+            hidden_states = torch.cat([hidden_states, encoder_hidden_states], dim=1)
+        heads = attn.heads
+        split = lambda t: t.unflatten(2, (heads, -1)).transpose(1, 2)       # [B, S, H*D] -> [B, H, S, D] view
+        table = rope_table_from_cos_sin(image_rotary_emb[0], image_rotary_emb[1], extra_tokens=n_text)
+        query = RMSNormRopeHeadsFunction.apply(split(attn.to_q(hidden_states)), attn.norm_q.weight, table, attn.norm_q.eps)
+        key = RMSNormRopeHeadsFunction.apply(split(attn.to_k(hidden_states)), attn.norm_k.weight, table, attn.norm_k.eps)
+        value = split(attn.to_v(hidden_states))
+        if attn.add_q_proj is not None and encoder_hidden_states is not None:
+            encoder_query = split(attn.add_q_proj(encoder_hidden_states))
+            encoder_key = split(attn.add_k_proj(encoder_hidden_states))
+            encoder_value = split(attn.add_v_proj(encoder_hidden_states))
+            if attn.norm_added_q is not None:
+                encoder_query = attn.norm_added_q(encoder_query)
+            if attn.norm_added_k is not None:
+                encoder_key = attn.norm_added_k(encoder_key)
+            query = torch.cat([query, encoder_query], dim=2)
+            key = torch.cat([key, encoder_key], dim=2)
+            value = torch.cat([value, encoder_value], dim=2)
+        if attention_mask is not None:
+            attention_mask = attention_mask.unsqueeze(dim=1)
+        hidden_states = F.scaled_dot_product_attention(query, key, value, attn_mask=attention_mask, dropout_p=0.0,
+                                                       is_causal=False)
+        hidden_states = hidden_states.transpose(1, 2).flatten(2, 3).to(query.dtype)
+        if encoder_hidden_states is not None:
+            n_enc = encoder_hidden_states.shape[1]
+            hidden_states, encoder_hidden_states = hidden_states[:, :-n_enc], hidden_states[:, -n_enc:]
+            if getattr(attn, "to_out", None) is not None:
+                hidden_states = attn.to_out[1](attn.to_out[0](hidden_states))
+            if getattr(attn, "to_add_out", None) is not None:
+                encoder_hidden_states = attn.to_add_out(encoder_hidden_states)
+        return hidden_states, encoder_hidden_states
 
 
 def _is_self_attention(m: nn.Module) -> bool:
@@ -233,7 +332,7 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
     ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
     tokens.  ``blocks`` also replaces the forward of whole DiT blocks (see the module docstring).
     Returns counts of what was swapped."""
-    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0, "attention": 0}
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0, "attention": 0, "processor": 0}
     for ns in namespaces:
         fn = getattr(ns, "modulate", None)
         if callable(fn) and not hasattr(fn, "__wrapped__"):
@@ -253,6 +352,16 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if blocks and rmsnorm and _is_self_attention(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_self_attention_forward, module)
             counts["attention"] += 1
+        if gate and type(module).__name__ in GATE_METHOD_OWNERS:
+            fn = getattr(module, "gate", None)
+            if (callable(fn) and not isinstance(fn, nn.Module) and not hasattr(fn, "__wrapped__")
+                    and not (_is_cp_callable("gate", fn) and _several_ranks())):
+                module.gate = fused_gate(fn)        # instance attribute: shadows the method, as parallel_model.py:241 does
+                counts["gate"] += 1
+        if blocks and rmsnorm and type(getattr(module, "processor", None)).__name__ == HUNYUAN_PROCESSOR \
+                and all(hasattr(module, a) for a in ("to_q", "to_k", "to_v", "heads", "norm_q", "norm_k", "add_q_proj")):
+            module.processor = FusedHunyuanAttnProcessor(module.processor)
+            counts["processor"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
             # The *_with_cp_grad_reduce callables all-reduce their parameter gradients over the
             # context-parallel group; they are only replaced where that is the identity.  An owner

@@ -1,0 +1,174 @@
+"""Writes tests/golden/model_inventory.json: the structure of the reference model classes that
+teletron_amd.swap_in patches (which sub-modules a class holds under which attribute, how its
+LayerNorms are constructed, which methods it has, what its forward calls, how the output of each
+normalisation is consumed, and what the context-parallel models assign onto their blocks).
+
+Runs in the build container only (it reads /root/reference):
+
+    python tests/golden/make_model_inventory.py [/root/reference]
+
+Sources and how they are read:
+  teletron/models/wan/wan_model.py            syntax tree of the source text, and additionally loaded by
+                                              file path (it needs only torch + einops) to instantiate
+                                              tiny DiTBlock / Head modules, whose real children are
+                                              recorded next to the syntax-tree view
+  teletron/models/wan/parallel_wan_model.py   syntax tree only (imports megatron)
+  teletron/models/hunyuan/model.py            syntax tree only (imports diffusers)
+  teletron/models/hunyuan/parallel_model.py   syntax tree only
+  teletron/core/context_parallel/layers.py    syntax tree only (imports megatron)
+The JSON holds names, literal constructor arguments and short expressions, no source text.
+"""
+import ast
+import importlib.util
+import json
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FILES = {
+    "wan": "teletron/models/wan/wan_model.py",
+    "wan_parallel": "teletron/models/wan/parallel_wan_model.py",
+    "hunyuan": "teletron/models/hunyuan/model.py",
+    "hunyuan_parallel": "teletron/models/hunyuan/parallel_model.py",
+    "cp_layers": "teletron/core/context_parallel/layers.py",
+}
+# classes whose structure matters to the swap (everything else in those files is left out)
+CLASSES = {
+    "wan": ["RMSNorm", "AttentionModule", "SelfAttention", "CrossAttention", "GateModule", "DiTBlock", "Head"],
+    "wan_parallel": ["ContextParallelWanDitBlock", "ParallelWanModel"],
+    "hunyuan": ["HunyuanVideoAttnProcessor2_0", "FP32LayerNorm", "AdaLayerNormZero", "AdaLayerNormZeroSingle",
+                "HunyuanVideoSingleTransformerBlock", "HunyuanVideoTransformerBlock"],
+    "hunyuan_parallel": ["HunyuanVideoDoubleAttnProcessor2_0", "HunyuanVideoSingleAttnProcessor2_0",
+                         "ParallelHunyuanVideoModel"],
+    "cp_layers": ["ContextParallelGateModule", "GateWithGradReduce", "ModulateWithCPGradReduce"],
+}
+FUNCTIONS = {"wan": ["modulate", "rope_apply"], "cp_layers": ["gate_with_cp_grad_reduce", "modulate_with_cp_grad_reduce"]}
+
+
+def dotted(node):
+    """`self.norm1` / `attn.to_q` / `modulate` for a call target; other expressions in short form."""
+    if isinstance(node, ast.Name):
+        return node.id
+    if isinstance(node, ast.Attribute):
+        return dotted(node.value) + "." + node.attr
+    return ast.unparse(node)
+
+
+def literal(node):
+    try:
+        return ast.literal_eval(node)
+    except Exception:
+        return ast.unparse(node)
+
+
+def parents_of(fn):
+    parent = {}
+    for n in ast.walk(fn):
+        for c in ast.iter_child_nodes(n):
+            parent[c] = n
+    return parent
+
+
+def consumer_of(node, parent, fn):
+    """How the value of the call `node` is used: 'call:<callee>' (passed as an argument), 'inline'
+    (left operand of a multiplication, the `norm(x) * (1 + scale) + shift` form), via one
+    intermediate variable if need be, else 'other'."""
+    p = parent.get(node)
+    if isinstance(p, ast.Call) and node in p.args:
+        return "call:" + dotted(p.func)
+    if isinstance(p, ast.BinOp) and isinstance(p.op, ast.Mult) and p.left is node:
+        return "inline"
+    if isinstance(p, ast.Assign) and len(p.targets) == 1 and isinstance(p.targets[0], ast.Name):
+        var = p.targets[0].id
+        later = [n for n in ast.walk(fn) if isinstance(n, ast.Name) and n.id == var and isinstance(n.ctx, ast.Load)
+                 and (n.lineno, n.col_offset) > (node.end_lineno, node.end_col_offset)]
+        if later:       # the first read of the variable in source order decides
+            return consumer_of(min(later, key=lambda n: (n.lineno, n.col_offset)), parent, fn)
+    return "other"
+
+
+def describe_class(cls):
+    out = {"bases": [dotted(b) for b in cls.bases], "children": [], "attributes": [], "methods": {}, "assignments": []}
+    for item in cls.body:
+        if not isinstance(item, ast.FunctionDef):
+            continue
+        out["methods"][item.name] = [a.arg for a in item.args.args]
+        if item.name == "__init__":
+            for n in ast.walk(item):
+                if not (isinstance(n, ast.Assign) and len(n.targets) == 1):
+                    continue
+                t, v = n.targets[0], n.value
+                if isinstance(t, ast.Attribute) and isinstance(t.value, ast.Name) and t.value.id == "self":
+                    if isinstance(v, ast.Call):
+                        out["children"].append({"attr": t.attr, "class": dotted(v.func).split(".")[-1],
+                                                "args": [literal(a) for a in v.args],
+                                                "kwargs": {k.arg: literal(k.value) for k in v.keywords if k.arg}})
+                    elif t.attr not in out["attributes"]:       # plain values: self.num_heads = num_heads
+                        out["attributes"].append(t.attr)
+                elif isinstance(t, ast.Attribute):      # assigned onto another object: self.blocks[i].gate = ...
+                    out["assignments"].append({"target": ast.unparse(t), "attr": t.attr, "value": ast.unparse(v)})
+        if item.name in ("forward", "__call__"):
+            parent = parents_of(item)
+            calls, uses = [], []
+            for n in ast.walk(item):
+                if isinstance(n, ast.Call):
+                    name = dotted(n.func)
+                    calls.append(name)
+                    if name.startswith("self.") and name.count(".") == 1:
+                        uses.append({"attr": name[5:], "consumer": consumer_of(n, parent, item)})
+            key = "forward" if item.name == "forward" else "call"
+            out[key + "_calls"] = sorted(set(calls))
+            out[key + "_uses_of_self_attributes"] = uses
+    return out
+
+
+def instantiate_wan(path):
+    """Tiny instances of the real classes: what named_children() really holds."""
+    spec = importlib.util.spec_from_file_location("reference_wan_model", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    import torch.nn as nn
+
+    def children(m):
+        d = {}
+        for name, c in m.named_children():
+            e = {"class": type(c).__name__}
+            if isinstance(c, nn.LayerNorm):
+                e.update(elementwise_affine=c.elementwise_affine, eps=c.eps)
+            if hasattr(c, "eps") and not isinstance(c, nn.LayerNorm):
+                e["eps"] = c.eps
+            d[name] = e
+        return d
+
+    blk = mod.DiTBlock(True, 64, 4, 128, 1e-6)
+    head = mod.Head(64, 4, (1, 2, 2), 1e-6)
+    return {"DiTBlock": {"children": children(blk), "parameters": [n for n, _ in blk.named_parameters(recurse=False)]},
+            "Head": {"children": children(head), "parameters": [n for n, _ in head.named_parameters(recurse=False)]},
+            "SelfAttention": {"children": children(blk.self_attn)},
+            "CrossAttention": {"children": children(blk.cross_attn)},
+            "RMSNorm": {"parameters": {n: list(p.shape) for n, p in blk.self_attn.norm_q.named_parameters()},
+                        "methods": sorted(n for n in ("norm", "forward") if hasattr(blk.self_attn.norm_q, n))}}
+
+
+def main():
+    root = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    inv = {"files": FILES}
+    for key, rel in FILES.items():
+        tree = ast.parse(open(os.path.join(root, rel)).read())
+        classes = {n.name: describe_class(n) for n in tree.body if isinstance(n, ast.ClassDef) and n.name in CLASSES[key]}
+        missing = set(CLASSES[key]) - set(classes)
+        if missing:
+            raise SystemExit(f"{rel}: classes not found: {sorted(missing)}")
+        funcs = {n.name: [a.arg for a in n.args.args] for n in tree.body
+                 if isinstance(n, ast.FunctionDef) and n.name in FUNCTIONS.get(key, [])}
+        inv[key] = {"classes": classes, "functions": funcs}
+    inv["wan_instantiated"] = instantiate_wan(os.path.join(root, FILES["wan"]))
+    out = os.path.join(HERE, "model_inventory.json")
+    with open(out, "w") as f:
+        json.dump(inv, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print("wrote", out)
+
+
+if __name__ == "__main__":
+    main()

@@ -143,7 +143,8 @@ def test_swap_in_matches_eager_model(monkeypatch):
     assert S.swap_in_if_requested(model, [ns]) is None
     monkeypatch.setenv("FUSED_KERNELS", "1")
     counts = S.swap_in_if_requested(model, [ns])
-    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4, "block": 0, "attention": 0}, counts
+    assert counts == {"rmsnorm": 4, "layernorm": 6, "modulate": 2, "gate": 4, "block": 0, "attention": 0,
+                      "processor": 0}, counts
     assert isinstance(model.blocks[0].norm3, nn.LayerNorm)               # affine LayerNorm untouched
     assert list(model.state_dict().keys()) == keys_before                 # checkpoint compatible
     try:
@@ -157,7 +158,8 @@ def test_swap_in_matches_eager_model(monkeypatch):
         assert rel(a, b) < 2e-2
     worst = max(rel(gp_f[n], gp_e[n]) for n in gp_e)
     assert worst < 2e-2, worst
-    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0, "block": 0, "attention": 0}   # idempotent on the model
+    assert S.swap_in(model, [ns]) == {"rmsnorm": 0, "layernorm": 0, "modulate": 1, "gate": 0, "block": 0, "attention": 0,
+                                     "processor": 0}   # idempotent on the model
 
 
 class RefAttention(nn.Module):
