@@ -50,6 +50,24 @@ def assert_grad_close(got, ref, rows_reduced, what):
     assert not bad.any(), f"{what}: {int(bad.sum())} of {ref.numel()} outside tolerance, worst err {float(err.max()):.3e}"
 
 
+def assert_grad_rtol(got, ref, rows_reduced, what):
+    """The parameter-gradient contract as the pure relative bound: on every column whose true sum is
+    not small against the random-walk size of a sum over `rows_reduced` O(1) terms
+    (|ref| >= 0.25 * sqrt(rows)), |got - ref| <= 1e-3 * |ref| with no absolute term.  Prints the
+    worst relative error on those columns and the share of all columns that only the absolute
+    term of assert_grad_close covers."""
+    got = got.detach().double().cpu().reshape(-1)
+    ref = ref.double().reshape(-1)
+    err = (got - ref).abs()
+    posed = ref.abs() >= 0.25 * math.sqrt(rows_reduced)
+    assert posed.any(), f"{what}: no column with a well-posed relative bound"
+    rel = (err[posed] / ref.abs()[posed]).max().item()
+    rescued = (err > 1e-3 * ref.abs()).double().mean().item()
+    print(f"[grad contract] {what}: {int(posed.sum())} of {ref.numel()} columns well-posed, worst relative error there "
+          f"{rel:.3e}; {100 * rescued:.2f} % of all columns rely on the absolute term")
+    assert rel <= 1e-3, f"{what}: relative error {rel:.3e} > 1e-3 on a well-posed column"
+
+
 def rand_bf16(*shape, seed, scale=1.0, offset=0.0):
     g = torch.Generator().manual_seed(seed)
     return (offset + scale * torch.randn(*shape, generator=g)).to(torch.bfloat16)
