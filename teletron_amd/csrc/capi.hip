@@ -115,7 +115,7 @@ constexpr int kMaxWgsPerCu = 8;
 
 // `res`: 0, or the residual + LayerNorm fusion: 1 plain, 2 gated (wide rows, kFwd / kBwd only).
 int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_batch, Plan* plan, bool rope = false,
-              int res = 0) {
+              int res = 0, int64_t rope_heads = 0) {
   if (rows <= 0 || cols <= 0 || rows_per_batch <= 0 || rows % rows_per_batch != 0)
     return TT_ERR_INVALID_ARGUMENT;
   if (cols > TT_MAX_COLS) return TT_ERR_UNSUPPORTED;
@@ -132,7 +132,7 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
     k = res == 2 ? resnorm_gated_kernel(dir == kBwd, idx, full) : resnorm_plain_kernel(dir == kBwd, idx, full);
   } else if (rope) {
     if (kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
-    k = rms_rope_kernel(narrow, dir == kBwd, idx, full);
+    k = rms_rope_kernel(narrow, dir == kBwd, idx, full, rope_heads);
   } else if (kind == kAdaLN)
     k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
@@ -215,11 +215,13 @@ size_t workspace_for(int kind, int n_acc, int64_t rows, int64_t cols, int64_t ro
     const size_t ns = partial_bytes(ps, n_acc, cols);
     if (ns > need) need = ns;
   }
-  if (kind == kRMS) {   // tt_rmsnorm_rope[_heads]_backward share this size query
-    Plan pr;
-    if (make_plan(kRMS, kBwd, rows, cols, rows, &pr, true) == TT_OK) {
-      const size_t nr = partial_bytes(pr, n_acc, cols);
-      if (nr > need) need = nr;
+  if (kind == kRMS) {   // tt_rmsnorm_rope[_heads]_backward share this size query: per-row and per-token kernels
+    for (int64_t heads : {(int64_t)0, (int64_t)kRopeTokenHeads}) {
+      Plan pr;
+      if (make_plan(kRMS, kBwd, rows, cols, rows, &pr, true, 0, heads) == TT_OK) {
+        const size_t nr = partial_bytes(pr, n_acc, cols);
+        if (nr > need) need = nr;
+      }
     }
   }
   return need < 16 ? 16 : need;
@@ -336,7 +338,7 @@ int forward(int kind, void* y, const void* x, const void* p0, const void* p1, fl
     return forward_generic(kind, y, x, p0, p1, mean, rstd, x_norm, rows, cols, rows_per_batch, eps, stream);
   }
   Plan p;
-  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p, rope != nullptr);
+  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p, rope != nullptr, 0, rope ? rope->heads : 0);
   if (rc != TT_OK) return rc;
   FwdArgs a;
   a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
@@ -360,7 +362,7 @@ int backward_partials(int kind, void* dx, const void* dy, const void* x, const v
     if (rrc != TT_OK) return rrc;
   }
   Plan p;
-  int rc = make_plan(kind, kBwd, rows, cols, rows_per_batch, &p, rope != nullptr);
+  int rc = make_plan(kind, kBwd, rows, cols, rows_per_batch, &p, rope != nullptr, 0, rope ? rope->heads : 0);
   if (rc != TT_OK) return rc;
   const int n_acc = kind == kAdaLN ? 2 : 1;
   if (!workspace || !aligned16(workspace) || workspace_bytes < partial_bytes(p, n_acc, cols)) return TT_ERR_WORKSPACE;

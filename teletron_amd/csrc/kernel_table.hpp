@@ -193,7 +193,27 @@ KernelInfo info_bwd_rope_narrow() {
   constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
   return {reinterpret_cast<const void*>(&norm_bwd_narrow<kRMS, L, R, NW, FULL, true>), 64 * NW, NW * R * (64 / L), R};
 }
-inline KernelInfo lookup_rope(bool narrow, bool backward, int idx, bool full) {
+// Token mode of the narrow ROPE kernels (ROPE = 2: the rows a wave takes per tile are the heads of
+// one token, so the (cos, sin) entries are loaded once per tile and lane).  Instantiated for rows of
+// 16 lanes (head_dim 72 ... 128) and 24 heads per token, HunyuanVideo's layout: 24 rows / 4 rows per
+// load = 6 loads per lane.
+constexpr int kRopeTokenL = 16, kRopeTokenR = 6, kRopeTokenHeads = kRopeTokenR * (64 / kRopeTokenL);
+#ifndef TT_ROPE_TOKEN_FWD_NW
+#define TT_ROPE_TOKEN_FWD_NW 4
+#endif
+#ifndef TT_ROPE_TOKEN_BWD_NW
+#define TT_ROPE_TOKEN_BWD_NW 4
+#endif
+template <bool FULL>
+KernelInfo info_rope_token(bool backward) {
+  constexpr int L = kRopeTokenL, R = kRopeTokenR, NF = TT_ROPE_TOKEN_FWD_NW, NB = TT_ROPE_TOKEN_BWD_NW;
+  if (backward)
+    return {reinterpret_cast<const void*>(&norm_bwd_narrow<kRMS, L, R, NB, FULL, 2>), 64 * NB, NB * R * (64 / L), R};
+  return {reinterpret_cast<const void*>(&norm_fwd_narrow<kRMS, L, R, NF, FULL, 2>), 64 * NF, NF * R * (64 / L), R};
+}
+inline KernelInfo lookup_rope(bool narrow, bool backward, int idx, bool full, int64_t heads) {
+  if (narrow && kNarrowL[idx] == kRopeTokenL && heads == kRopeTokenHeads)
+    return full ? info_rope_token<true>(backward) : info_rope_token<false>(backward);
   if (narrow) {
     switch (idx) {
 #define X(i, L)                                                                                       \
@@ -321,7 +341,7 @@ KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_saved_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_saved_kernel(bool narrow, int idx, bool full);
-KernelInfo rms_rope_kernel(bool narrow, bool backward, int idx, bool full);
+KernelInfo rms_rope_kernel(bool narrow, bool backward, int idx, bool full, int64_t heads);
 KernelInfo gate_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo gate_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo resnorm_plain_kernel(bool backward, int idx, bool full);

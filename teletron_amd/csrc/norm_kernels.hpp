@@ -551,10 +551,14 @@ struct RowPos {
 // ============================================================================ narrow forward
 // L lanes per row (one pack each), 64/L rows per wave per load, R loads in flight,
 // NW independent waves per workgroup.  A tile is NW*R*(64/L) consecutive rows.
-template <int KIND, int L, int R, int NW, bool FULL, bool ROPE = false>
+// ROPE: 0 none; 1 every row looks up its own position; 2 the R * 64/L rows a wave takes per tile
+// are exactly the heads of ONE token (the caller guarantees rows_per_pos == R * 64/L), so a lane
+// loads its (cos, sin) entries once per tile instead of once per row.
+template <int KIND, int L, int R, int NW, bool FULL, int ROPE = 0>
 __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
   static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
+  constexpr int NF = ROPE == 1 ? R : 1;   // table entries held per lane
   constexpr int RPW = 64 / L;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -583,12 +587,12 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
 
   u32x4 raw[R];
   // ROPE: the 4 (cos, sin) pairs of this lane's pack at the row's position travel with the row.
-  float fr[ROPE ? R : 1][8];
-  RowPos rp[ROPE ? R : 1];
+  float fr[NF][8];
+  RowPos rp[NF];
   if constexpr (ROPE) {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri + r * RPW,
+    for (int r = 0; r < NF; ++r)
+      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + (ROPE == 1 ? ri + r * RPW : 0),
                  (int64_t)gridDim.x * (NW * R * RPW), a.rows_per_pos, a.seq_len);
   }
   auto fetch = [&](int64_t t) {
@@ -598,14 +602,20 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
       const int64_t rr = rb + r * RPW;
       raw[r] = u32x4{0, 0, 0, 0};
       if constexpr (ROPE) {
+        if (r < NF) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) fr[r][j] = 0.f;
+          for (int j = 0; j < 8; ++j) fr[r < NF ? r : 0][j] = 0.f;
+        }
       }
       if (rr < S && act) {
         raw[r] = load_stream(a.x, (size_t)((b * S + rr) * C + col));
-        if constexpr (ROPE) load_freq8(a.freqs, (size_t)(rp[r].pos * a.head_dim + col), fr[r]);
+        if constexpr (ROPE) {
+          if (r < NF) load_freq8(a.freqs, (size_t)(rp[r < NF ? r : 0].pos * a.head_dim + col), fr[r < NF ? r : 0]);
+        }
       }
-      if constexpr (ROPE) rp[r].advance(a.rows_per_pos, a.seq_len);
+      if constexpr (ROPE) {
+        if (r < NF) rp[r < NF ? r : 0].advance(a.rows_per_pos, a.seq_len);
+      }
     }
   };
 
@@ -614,7 +624,7 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   for (; tile < a.n_tiles; tile += gridDim.x) {
     const int64_t rbase = tile * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri;
     float xf[R][8];
-    float fc[ROPE ? R : 1][8];
+    float fc[NF][8];
     bool rv[R];
     if (!PF) fetch(tile);
 #pragma unroll
@@ -622,8 +632,10 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
       rv[r] = rbase + r * RPW < S;
       unpack8(raw[r], xf[r]);
       if constexpr (ROPE) {
+        if (r < NF) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) fc[r][j] = fr[r][j];
+          for (int j = 0; j < 8; ++j) fc[r < NF ? r : 0][j] = fr[r < NF ? r : 0][j];
+        }
       }
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
@@ -658,7 +670,7 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
           n[j] = xh;
           o[j] = ADALN ? fmaf(xh, g[j], sh[j]) : xh * g[j];
         }
-        if constexpr (ROPE) rope_rotate(o, fc[r]);
+        if constexpr (ROPE) rope_rotate(o, fc[ROPE == 1 ? r : 0]);
         store_stream(a.y, (size_t)(row * C + col), pack8(o));
         if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col), pack8(n));
         if (pi == 0) {
@@ -707,10 +719,11 @@ __device__ __forceinline__ void narrow_write_partials(float (&acc0)[8], float (&
 }
 
 // ============================================================================ narrow backward
-template <int KIND, int L, int R, int NW, bool FULL, bool ROPE = false>
+template <int KIND, int L, int R, int NW, bool FULL, int ROPE = 0>   // ROPE as in norm_fwd_narrow
 __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
   static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
+  constexpr int NF = ROPE == 1 ? R : 1;
   constexpr int NACC = ADALN ? 2 : 1;
   constexpr int RPW = 64 / L;
 
@@ -738,12 +751,12 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
   }
 
   u32x4 rawx[R], rawd[R];
-  float fr[ROPE ? R : 1][8];   // as in the forward kernel
-  RowPos rp[ROPE ? R : 1];
+  float fr[NF][8];   // as in the forward kernel
+  RowPos rp[NF];
   if constexpr (ROPE) {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + ri + r * RPW,
+    for (int r = 0; r < NF; ++r)
+      rp[r].init(b * S + (int64_t)blockIdx.x * (NW * R * RPW) + (int64_t)wave * (R * RPW) + (ROPE == 1 ? ri + r * RPW : 0),
                  (int64_t)gridDim.x * (NW * R * RPW), a.rows_per_pos, a.seq_len);
   }
   auto fetch = [&](int64_t t) {
@@ -754,16 +767,22 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       rawx[r] = u32x4{0, 0, 0, 0};
       rawd[r] = u32x4{0, 0, 0, 0};
       if constexpr (ROPE) {
+        if (r < NF) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) fr[r][j] = 0.f;
+          for (int j = 0; j < 8; ++j) fr[r < NF ? r : 0][j] = 0.f;
+        }
       }
       if (rr < S && act) {
         const size_t off = (size_t)((b * S + rr) * C + col);
         rawx[r] = load_stream(a.x, off);
         rawd[r] = load_stream(a.dy, off);
-        if constexpr (ROPE) load_freq8(a.freqs, (size_t)(rp[r].pos * a.head_dim + col), fr[r]);
+        if constexpr (ROPE) {
+          if (r < NF) load_freq8(a.freqs, (size_t)(rp[r < NF ? r : 0].pos * a.head_dim + col), fr[r < NF ? r : 0]);
+        }
       }
-      if constexpr (ROPE) rp[r].advance(a.rows_per_pos, a.seq_len);
+      if constexpr (ROPE) {
+        if (r < NF) rp[r < NF ? r : 0].advance(a.rows_per_pos, a.seq_len);
+      }
     }
   };
 
@@ -780,7 +799,7 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       unpack8(rawx[r], xf[r]);
       unpack8(rawd[r], df[r]);
       // the incoming gradient is that of the rotated output: undo the rotation first
-      if constexpr (ROPE) rope_unrotate(df[r], fr[r]);
+      if constexpr (ROPE) rope_unrotate(df[r], fr[ROPE == 1 ? r : 0]);
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
     if constexpr (NW > 1) __syncthreads();   // lock-step only: keeps the request stream narrow (+1-2 %)

@@ -3,5 +3,7 @@
 #include "kernel_table.hpp"
 
 namespace tt {
-KernelInfo rms_rope_kernel(bool narrow, bool backward, int idx, bool full) { return lookup_rope(narrow, backward, idx, full); }
+KernelInfo rms_rope_kernel(bool narrow, bool backward, int idx, bool full, int64_t heads) {
+  return lookup_rope(narrow, backward, idx, full, heads);
+}
 }  // namespace tt
