@@ -676,7 +676,9 @@ int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void*
   // mix on MI355X (reads want many requests in flight, writes few: 4 waves with one store each).
   const int threads = !a ? 256 : kProbeMaxThreads;
   const size_t want = (n + threads - 1) / threads;
-  const dim3 grid((unsigned)(want < (size_t)cus ? want : (size_t)cus));
+  // two reads per write stream best with one CU in 32 left without a workgroup, like the kernels
+  const size_t wgs = (b && cus >= 32) ? (size_t)(cus - cus / 32) : (size_t)cus;
+  const dim3 grid((unsigned)(want < wgs ? want : wgs));
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!out)    hipLaunchKernelGGL((stream_probe<kProbeRead, 4>), grid, dim3(threads), 0, s, out, a, b, n);
   else if (!a) hipLaunchKernelGGL((stream_probe<kProbeWrite, 1>), grid, dim3(threads), 0, s, out, a, b, n);

@@ -26,15 +26,11 @@ __device__ __forceinline__ u32x4 load_stream(const void* base, size_t elem_off) 
 }
 __device__ __forceinline__ void store_stream(void* base, size_t elem_off, u32x4 v) {
   u32x4* p = reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + elem_off);
-#if defined(TT_STORE_NT)
-  __builtin_nontemporal_store(v, p);
-#else
   // The compiler pads its own stores wider than 64 bits against two hazards of this target but
   // cannot see inside the asm, so the padding is spelled out: two wait states between a VALU
   // write of the data registers and the store, and two between the store and the next VALU
   // write of those registers (the data is read after issue).  Four are spent on each side.
   asm volatile("s_nop 3\n\tglobal_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 3" ::"v"(p), "v"(v) : "memory");
-#endif
 }
 __device__ __forceinline__ u32x4 load_cached(const void* base, size_t elem_off) {
   return *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + elem_off);

@@ -37,26 +37,13 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 // roughly 18 (forward) / 12 (backward, two input tensors) outstanding 128-bit loads per lane
 // column of a CU and tensor, and barrier-coupled row groups in ONE workgroup per CU stream
 // better than independent workgroups; Q is chosen so that one workgroup carries that load.
-#ifndef TT_FWD_R
-#define TT_FWD_R 1
-#endif
-#ifndef TT_BWD_R
-#define TT_BWD_R 1
-#endif
-#ifndef TT_NARROW_FWD_R
-#define TT_NARROW_FWD_R 2
-#endif
-#ifndef TT_NARROW_BWD_R
-#define TT_NARROW_BWD_R 2
-#endif
-#ifndef TT_NARROW_NW
-#define TT_NARROW_NW 4
-#endif
+constexpr int kNarrowR = 2;    // loads per lane and tensor in flight, narrow kernels (3 ... 8 measured within 1 %)
+constexpr int kNarrowNW = 4;   // independent waves per workgroup, narrow kernels
 constexpr int kFwdLoadsPerCu = 18;   // target waves x loads-per-lane per CU, forward
 constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
 
-constexpr int fwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_FWD_R; }
-constexpr int bwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_BWD_R; }
+constexpr int fwd_wide_R(int W, int P) { return 1; }   // two rows per tile: 1-3 % slower at every width
+constexpr int bwd_wide_R(int W, int P) { return 1; }
 // AdaLN backward has two barrier-coupled reductions per row; on the variants below two rows per
 // row group and tile (both rows share each exchange) hide that latency better.  Measured,
 // us at R = 1 -> R = 2: 32760 x 1536: 53.8 -> 51.9; 4 x 32760 x 1536: 200.8 -> 198.0;
@@ -65,29 +52,17 @@ constexpr int bwd_wide_R(int W, int P) { return P >= 4 ? 1 : TT_BWD_R; }
 // (356.6 -> 368.8), 8192 (358.0 -> 399.5), and 5120 (ten waves: spills).  RMSNorm (one reduction
 // per row) is 2-3 % slower with R = 2 everywhere.
 constexpr int adaln_bwd_wide_R(int W, int P) {
-#ifdef TT_ADALN_BWD_R
-  return P >= 4 ? 1 : TT_ADALN_BWD_R;
-#else
   return ((P == 1 && W >= 2 && W <= 4) || (P == 2 && (W == 3 || W == 6))) ? 2 : bwd_wide_R(W, P);
-#endif
 }
 constexpr int fwd_wide_Q(int W, int P) {
-#ifdef TT_FWD_Q
-  return TT_FWD_Q * W > 16 ? 1 : TT_FWD_Q;
-#else
   return W >= 7 ? 1 : (10 + W / 2) / W;          // about 10 waves per workgroup
-#endif
 }
 constexpr int bwd_wide_Q(int W, int P) {
-#ifdef TT_BWD_Q
-  return TT_BWD_Q * W > 16 ? 1 : TT_BWD_Q;
-#else
   int q = (2 * kBwdLoadsPerCu + W * P) / (2 * W * P);   // round(12 / (W*P))
   if (q < 1) q = 1;
   if (W * q < 6) q = (6 + W - 1) / W;                   // at least 6 waves to keep up with the arithmetic
   while (q > 1 && W * q > 12) --q;                      // at most 12 waves: 170 VGPRs per lane
   return q;
-#endif
 }
 
 // Index of the wide variant for `packs` (> kNarrowMaxPacks), or -1.
@@ -123,17 +98,17 @@ KernelInfo info_bwd_saved_wide() {
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_saved_narrow() {
-  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_saved_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_fwd_narrow() {
-  constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_fwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_narrow() {
-  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 
@@ -185,12 +160,12 @@ KernelInfo info_bwd_rope_wide() {
 }
 template <int L, bool FULL>
 KernelInfo info_fwd_rope_narrow() {
-  constexpr int R = TT_NARROW_FWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_fwd_narrow<kRMS, L, R, NW, FULL, true>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int L, bool FULL>
 KernelInfo info_bwd_rope_narrow() {
-  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_narrow<kRMS, L, R, NW, FULL, true>), 64 * NW, NW * R * (64 / L), R};
 }
 // Token mode of the narrow ROPE kernels (ROPE = 2: the rows a wave takes per tile are the heads of
@@ -198,15 +173,13 @@ KernelInfo info_bwd_rope_narrow() {
 // 16 lanes (head_dim 72 ... 128) and 24 heads per token, HunyuanVideo's layout: 24 rows / 4 rows per
 // load = 6 loads per lane.
 constexpr int kRopeTokenL = 16, kRopeTokenR = 6, kRopeTokenHeads = kRopeTokenR * (64 / kRopeTokenL);
-#ifndef TT_ROPE_TOKEN_FWD_NW
-#define TT_ROPE_TOKEN_FWD_NW 4
-#endif
-#ifndef TT_ROPE_TOKEN_BWD_NW
-#define TT_ROPE_TOKEN_BWD_NW 4
-#endif
+// Four waves in one workgroup per CU (24 loads per lane column and tensor in flight) measured best:
+// forward 245 us, backward + reduction 356 us at 118800 x 24 x 128; 5 / 6 / 8 waves: 277 / 265 / 267 us
+// forward, 378 / 368 / 380 us backward; 2 and 3 waves need 2-3 workgroups per CU and reach 259-265 us.
+constexpr int kRopeTokenNW = 4;
 template <bool FULL>
 KernelInfo info_rope_token(bool backward) {
-  constexpr int L = kRopeTokenL, R = kRopeTokenR, NF = TT_ROPE_TOKEN_FWD_NW, NB = TT_ROPE_TOKEN_BWD_NW;
+  constexpr int L = kRopeTokenL, R = kRopeTokenR, NF = kRopeTokenNW, NB = kRopeTokenNW;
   if (backward)
     return {reinterpret_cast<const void*>(&norm_bwd_narrow<kRMS, L, R, NB, FULL, 2>), 64 * NB, NB * R * (64 / L), R};
   return {reinterpret_cast<const void*>(&norm_fwd_narrow<kRMS, L, R, NF, FULL, 2>), 64 * NF, NF * R * (64 / L), R};
@@ -243,7 +216,7 @@ KernelInfo info_gate_wide() {
 }
 template <int MODE, int L, bool FULL>
 KernelInfo info_gate_narrow() {
-  constexpr int R = TT_NARROW_BWD_R, NW = TT_NARROW_NW;
+  constexpr int R = kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&gate_narrow<MODE, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int MODE>
@@ -279,18 +252,10 @@ constexpr int res_waves_Q(int W, int P) {
   return q < 1 ? 1 : q;
 }
 constexpr int res_fwd_Q(int W, int P) {
-#ifdef TT_RES_FWD_Q
-  return TT_RES_FWD_Q * W > 16 ? 1 : TT_RES_FWD_Q;
-#else
   return res_waves_Q(W, P);
-#endif
 }
 constexpr int res_bwd_Q(int W, int P, bool gated) {
-#ifdef TT_RES_BWD_Q
-  return TT_RES_BWD_Q * W > 16 ? 1 : TT_RES_BWD_Q;
-#else
   return res_waves_Q(W, P);
-#endif
 }
 template <int W, int P, bool FULL, bool GATED>
 KernelInfo info_res_fwd() {
