@@ -90,7 +90,8 @@ def test_rope_full_size_rows_and_reproducibility():
 
 # ---------------------------------------------------------------- per-head norm + rotary (HunyuanVideo layout)
 @pytest.mark.parametrize("b,s,heads,hd", [(1, 1, 1, 128), (2, 37, 24, 128), (1, 301, 3, 64), (3, 19, 5, 8), (1, 50, 7, 72),
-                                          (1, 23, 4, 256), (2, 1000, 2, 32), (2, 53, 12, 128), (1, 200, 6, 128)])
+                                          (1, 23, 4, 256), (2, 1000, 2, 32), (2, 53, 12, 128), (1, 200, 6, 128),
+                                          (2, 31, 24, 72), (1, 45, 24, 104), (3, 1, 24, 128)])   # 24 heads: one token per wave and tile
 def test_rmsnorm_rope_heads_shapes(b, s, heads, hd):
     from teletron_amd import ops
     seed = 1000 + hd + s
