@@ -37,7 +37,12 @@ constexpr int kMaxPacks = 64 * 16 * 4;
 // roughly 18 (forward) / 12 (backward, two input tensors) outstanding 128-bit loads per lane
 // column of a CU and tensor, and barrier-coupled row groups in ONE workgroup per CU stream
 // better than independent workgroups; Q is chosen so that one workgroup carries that load.
-constexpr int kNarrowR = 2;    // loads per lane and tensor in flight, narrow kernels (3 ... 8 measured within 1 %)
+constexpr int kNarrowR = 2;    // loads per lane and tensor in flight, narrow kernels
+// RMSNorm backward on narrow rows streams better with six loads per lane in ONE four-wave workgroup
+// per CU than with two loads in two workgroups: 2,851,200 x 128 backward 362 -> 354 us between
+// forward launches (reference contract 371 -> 358 us), 1-1.5 % at 32, 64 and 256 columns.  Forward
+// and the AdaLN kernels lose with six (128 columns forward 242 -> 269 us, AdaLN backward 359 -> 363 us).
+constexpr int kNarrowRmsBwdR = 6;
 constexpr int kNarrowNW = 4;   // independent waves per workgroup, narrow kernels
 constexpr int kFwdLoadsPerCu = 18;   // target waves x loads-per-lane per CU, forward
 constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
@@ -98,7 +103,7 @@ KernelInfo info_bwd_saved_wide() {
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_saved_narrow() {
-  constexpr int R = kNarrowR, NW = kNarrowNW;
+  constexpr int R = KIND == kRMS ? kNarrowRmsBwdR : kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_saved_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int KIND, int L, bool FULL>
@@ -108,7 +113,7 @@ KernelInfo info_fwd_narrow() {
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_narrow() {
-  constexpr int R = kNarrowR, NW = kNarrowNW;
+  constexpr int R = KIND == kRMS ? kNarrowRmsBwdR : kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 
