@@ -598,21 +598,17 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
     for (int r = 0; r < R; ++r) {
       const int64_t rr = rb + r * RPW;
       raw[r] = u32x4{0, 0, 0, 0};
-      if constexpr (ROPE) {
-        if (r < NF) {
+      const bool table = ROPE == 1 || (ROPE == 2 && r == 0);   // this load carries table entries with it
+      const int f = ROPE == 1 ? r : 0;
+      if (table) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) fr[r < NF ? r : 0][j] = 0.f;
-        }
+        for (int j = 0; j < 8; ++j) fr[f][j] = 0.f;
       }
       if (rr < S && act) {
         raw[r] = load_stream(a.x, (size_t)((b * S + rr) * C + col));
-        if constexpr (ROPE) {
-          if (r < NF) load_freq8(a.freqs, (size_t)(rp[r < NF ? r : 0].pos * a.head_dim + col), fr[r < NF ? r : 0]);
-        }
+        if (table) load_freq8(a.freqs, (size_t)(rp[f].pos * a.head_dim + col), fr[f]);
       }
-      if constexpr (ROPE) {
-        if (r < NF) rp[r < NF ? r : 0].advance(a.rows_per_pos, a.seq_len);
-      }
+      if (table) rp[f].advance(a.rows_per_pos, a.seq_len);
     }
   };
 
@@ -628,11 +624,9 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
     for (int r = 0; r < R; ++r) {
       rv[r] = rbase + r * RPW < S;
       unpack8(raw[r], xf[r]);
-      if constexpr (ROPE) {
-        if (r < NF) {
+      if (ROPE == 1 || (ROPE == 2 && r == 0)) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) fc[r < NF ? r : 0][j] = fr[r < NF ? r : 0][j];
-        }
+        for (int j = 0; j < 8; ++j) fc[ROPE == 1 ? r : 0][j] = fr[ROPE == 1 ? r : 0][j];
       }
     }
     if (PF && tile + gridDim.x < a.n_tiles) fetch(tile + gridDim.x);
@@ -763,23 +757,19 @@ __global__ __launch_bounds__(64 * NW) void norm_bwd_narrow(const BwdArgs a) {
       const int64_t rr = rb + r * RPW;
       rawx[r] = u32x4{0, 0, 0, 0};
       rawd[r] = u32x4{0, 0, 0, 0};
-      if constexpr (ROPE) {
-        if (r < NF) {
+      const bool table = ROPE == 1 || (ROPE == 2 && r == 0);   // as in the forward kernel
+      const int f = ROPE == 1 ? r : 0;
+      if (table) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) fr[r < NF ? r : 0][j] = 0.f;
-        }
+        for (int j = 0; j < 8; ++j) fr[f][j] = 0.f;
       }
       if (rr < S && act) {
         const size_t off = (size_t)((b * S + rr) * C + col);
         rawx[r] = load_stream(a.x, off);
         rawd[r] = load_stream(a.dy, off);
-        if constexpr (ROPE) {
-          if (r < NF) load_freq8(a.freqs, (size_t)(rp[r < NF ? r : 0].pos * a.head_dim + col), fr[r < NF ? r : 0]);
-        }
+        if (table) load_freq8(a.freqs, (size_t)(rp[f].pos * a.head_dim + col), fr[f]);
       }
-      if constexpr (ROPE) {
-        if (r < NF) rp[r < NF ? r : 0].advance(a.rows_per_pos, a.seq_len);
-      }
+      if (table) rp[f].advance(a.rows_per_pos, a.seq_len);
     }
   };
 
