@@ -35,8 +35,9 @@ ships no code that performs the swap.  This module does it by patching *instance
 * HunyuanVideo (``teletron/models/hunyuan/model.py``): ``norm2`` / ``norm2_context`` of
   ``HunyuanVideoTransformerBlock`` with the inline modulation after them (``:615-623,660-669``) go
   the token way as well; the ``gate(self, x, gate, residual)`` *methods* of both block classes
-  (``:538-539,627-628``) are shadowed by the fused gated residual add; with ``blocks=True`` every
-  attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
+  (``:538-539,627-628``) are shadowed by the fused gated residual add; with ``blocks=True`` the
+  double-stream block gets a ``forward`` that fuses its first gate with ``norm2`` + modulation
+  (:func:`fused_hunyuan_block_forward`) and every attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
   :class:`FusedHunyuanAttnProcessor`, which runs ``norm_q`` / ``norm_k`` and the rotary embedding
   after them as one kernel per tensor (text tokens appended to the latent ones take no rotation).
 
@@ -312,6 +313,43 @@ class FusedHunyuanAttnProcessor:
         return hidden_states, encoder_hidden_states
 
 
+def fused_hunyuan_block_forward(self, hidden_states, encoder_hidden_states, temb, attention_mask=None, freqs_cis=None):
+    """``HunyuanVideoTransformerBlock.forward`` (``hunyuan/model.py:630-681``) with the gated residual
+    update of the latent stream fused with the ``norm2`` + inline modulation that reads its result
+    (``:655-664``): one pass over the stream instead of two.  Everything else (``norm1`` /
+    ``norm1_context``, the attention, the feed-forwards, the text stream, the second gate) runs
+    through the block's own, possibly swapped, sub-modules in the reference's order."""
+    norm_hidden_states, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.norm1(hidden_states, emb=temb)
+    norm_encoder_hidden_states, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = self.norm1_context(
+        encoder_hidden_states, emb=temb)
+    attn_output, context_attn_output = self.attn(hidden_states=norm_hidden_states,
+                                                 encoder_hidden_states=norm_encoder_hidden_states,
+                                                 attention_mask=attention_mask, image_rotary_emb=freqs_cis)
+    if (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and attn_output.dtype == torch.bfloat16
+            and _same_dtype(hidden_states, gate_msa, shift_mlp, scale_mlp)):
+        hidden_states, norm_hidden_states = residual_adaln(hidden_states, attn_output, gate_msa.unsqueeze(1),
+                                                           shift_mlp[:, None], scale_mlp[:, None], self.norm2.eps)
+    else:
+        hidden_states = self.gate(hidden_states, gate_msa.unsqueeze(1), attn_output)
+        norm_hidden_states = self.norm2(hidden_states) * (1 + scale_mlp[:, None]) + shift_mlp[:, None]
+    encoder_hidden_states = encoder_hidden_states + context_attn_output * c_gate_msa.unsqueeze(1)
+    norm_encoder_hidden_states = self.norm2_context(encoder_hidden_states) * (1 + c_scale_mlp[:, None]) + c_shift_mlp[:, None]
+    ff_output = self.ff(norm_hidden_states)
+    context_ff_output = self.ff_context(norm_encoder_hidden_states)
+    hidden_states = self.gate(hidden_states, gate_mlp.unsqueeze(1), ff_output)
+    encoder_hidden_states = encoder_hidden_states + c_gate_mlp.unsqueeze(1) * context_ff_output
+    return hidden_states, encoder_hidden_states
+
+
+def _is_hunyuan_double_block(m: nn.Module) -> bool:
+    if type(m).__name__ != "HunyuanVideoTransformerBlock":
+        return False
+    if _several_ranks() and _is_cp_callable("gate", getattr(m, "gate", None)):
+        return False      # that gate all-reduces its gradient over the context-parallel group
+    return (all(hasattr(m, a) for a in ("norm1", "norm1_context", "attn", "ff", "ff_context", "gate"))
+            and all(hasattr(getattr(m, a, None), "eps") for a in ("norm2", "norm2_context")))
+
+
 def _is_self_attention(m: nn.Module) -> bool:
     return (type(m).__name__ == "SelfAttention" and all(hasattr(m, a) for a in ("q", "k", "v", "o", "attn", "num_heads"))
             and _is_rmsnorm(getattr(m, "norm_q", None)) and _is_rmsnorm(getattr(m, "norm_k", None)))
@@ -348,6 +386,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
             counts["gate"] += 1
         if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_dit_block_forward, module)
+            counts["block"] += 1
+        if blocks and adaln and gate and _is_hunyuan_double_block(module) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(fused_hunyuan_block_forward, module)
             counts["block"] += 1
         if blocks and rmsnorm and _is_self_attention(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_self_attention_forward, module)

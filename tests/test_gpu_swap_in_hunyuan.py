@@ -42,21 +42,22 @@ class WithRotary(nn.Module):
         return self.model(h, e, temb, *self.rotary)
 
 
-def test_hunyuan_swap_in_matches_eager_model():
+@pytest.mark.parametrize("head_dim", [128, 64])     # hidden 512: the residual + norm pair runs fused; 256: as its two halves
+def test_hunyuan_swap_in_matches_eager_model(head_dim):
     from teletron_amd import swap_in as S
-    model, inputs, rotary, dy = make_model_and_inputs()
+    model, inputs, rotary, dy = make_model_and_inputs(head_dim=head_dim)
     wrapped = WithRotary(model, rotary)
     keys_before = list(wrapped.state_dict().keys())
     out_e, gin_e, gp_e = run(wrapped, inputs, dy)
     counts = S.swap_in(wrapped, blocks=True)
     # LayerNorms: norm1.norm, norm1_context.norm, norm2, norm2_context, single norm.norm; modulate attributes of
     # the three AdaLayerNormZero[Single]; the gate method of each block; q/k (+ added q/k) RMSNorms; two processors
-    assert counts == {"rmsnorm": 6, "layernorm": 5, "modulate": 3, "gate": 2, "block": 0, "attention": 0,
+    assert counts == {"rmsnorm": 6, "layernorm": 5, "modulate": 3, "gate": 2, "block": 1, "attention": 0,
                       "processor": 2}, counts
     dbl, sgl = model.transformer_blocks[0], model.single_transformer_blocks[0]
     assert isinstance(dbl.norm2, S.DeferredLayerNorm) and isinstance(dbl.norm2_context, S.DeferredLayerNorm)
     assert isinstance(dbl.attn.processor, S.FusedHunyuanAttnProcessor) and isinstance(sgl.attn.processor, S.FusedHunyuanAttnProcessor)
-    assert "gate" in dbl.__dict__ and "gate" in sgl.__dict__
+    assert "gate" in dbl.__dict__ and "gate" in sgl.__dict__ and "forward" in dbl.__dict__
     assert list(wrapped.state_dict().keys()) == keys_before
     out_f, gin_f, gp_f = run(wrapped, inputs, dy)
     assert rel(out_f, out_e) < 5e-3, rel(out_f, out_e)

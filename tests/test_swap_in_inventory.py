@@ -137,7 +137,8 @@ def patched_sites(root, before):
             got[path] = "adaln"
         elif "forward" in m.__dict__:
             kind = {"RMSNorm": "rmsnorm", "GateModule": "gate-module", "ContextParallelGateModule": "gate-module",
-                    "DiTBlock": "block", "ContextParallelWanDitBlock": "block", "SelfAttention": "attention"}
+                    "DiTBlock": "block", "ContextParallelWanDitBlock": "block", "SelfAttention": "attention",
+                    "HunyuanVideoTransformerBlock": "block"}
             got[path] = kind.get(type(m).__name__, "unexpected forward on " + type(m).__name__)
         if hasattr(m.__dict__.get("gate"), "__wrapped__"):
             got[path + "#gate"] = "gate-method"
@@ -196,7 +197,8 @@ def test_swap_in_patches_every_recorded_site_and_nothing_else(blocks):
     counts = S.swap_in(root, [ns], blocks=blocks)
     got = patched_sites(root, before)
     if blocks:
-        want.update({"m0": "block", "m0.self_attn": "attention", "m2.attn#processor": "processor", "m3.attn#processor": "processor"})
+        want.update({"m0": "block", "m2": "block", "m0.self_attn": "attention", "m2.attn#processor": "processor",
+                     "m3.attn#processor": "processor"})
     assert got == want, sorted(set(got.items()) ^ set(want.items()))
     assert hasattr(ns.modulate, "__wrapped__")                 # DiTBlock calls the module-level modulate
     assert isinstance(root.m0.norm3, nn.LayerNorm)             # the affine norm3 stays
@@ -239,10 +241,29 @@ def test_context_parallel_assignments_are_recognised(monkeypatch):
     counts = S.swap_in(root, blocks=True)
     assert counts["processor"] == 0                            # the context-parallel processors are not replaced
     assert counts["gate"] == 2 + 1 + 2 and counts["modulate"] == 3 + 1, counts      # methods + CP callable + GateModules
-    assert counts["block"] == 1
+    assert counts["block"] == 2          # the Wan block and the double-stream block, both on one rank
     root = assigned_model()
     monkeypatch.setattr(S, "_several_ranks", lambda: True)
     counts = S.swap_in(root, blocks=True)
     assert counts["gate"] == 2 and counts["modulate"] == 1 and counts["block"] == 0, counts   # GateModules of the Wan block; norm1_context
     assert isinstance(root.m2.norm1, nn.LayerNorm) and isinstance(root.m0.norm1.norm, nn.LayerNorm)
     assert isinstance(root.m0.norm2, S.DeferredLayerNorm)      # inline modulation: row-local, no all-reduce involved
+
+
+def test_replacement_forwards_keep_the_recorded_signatures():
+    """Each forward / processor that swap_in installs takes the parameters, in order and by name, that
+    the reference's own method takes (callers pass some of them by keyword)."""
+    import inspect
+    pairs = [(S.fused_dit_block_forward, spec_of("DiTBlock")["methods"]["forward"]),
+             (S.fused_dit_block_forward, spec_of("ContextParallelWanDitBlock")["methods"]["forward"]),
+             (S.fused_self_attention_forward, spec_of("SelfAttention")["methods"]["forward"]),
+             (S.fused_hunyuan_block_forward, spec_of("HunyuanVideoTransformerBlock")["methods"]["forward"]),
+             (S.FusedHunyuanAttnProcessor.__call__, spec_of("HunyuanVideoAttnProcessor2_0")["methods"]["__call__"]),
+             (S._fused_gate_forward, spec_of("GateModule")["methods"]["forward"]),
+             (S._fused_rmsnorm_forward, spec_of("RMSNorm")["methods"]["forward"])]
+    for fn, recorded in pairs:
+        assert list(inspect.signature(fn).parameters) == recorded, (fn.__name__, recorded)
+    # the calls inside the double-stream block pass these by keyword
+    calls = spec_of("HunyuanVideoTransformerBlock")["forward_calls"]
+    assert {"self.norm1", "self.norm1_context", "self.attn", "self.norm2", "self.norm2_context", "self.ff",
+            "self.ff_context", "self.gate"} <= set(calls)
