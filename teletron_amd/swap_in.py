@@ -246,6 +246,27 @@ def fused_self_attention_forward(self, x, freqs):
     return self.o(self.attn(q, k, self.v(x)))
 
 
+class _RotaryTableCache:
+    """The fp32 (cos, sin) table of ``rope_table_from_cos_sin`` for the rotary pair a model hands to
+    all of its blocks in one forward pass: built on first use, reused while the very same tensor
+    objects (held weakly) are passed again unmodified.  One entry per number of appended text tokens."""
+
+    def __init__(self):
+        self.entries = {}
+
+    def get(self, cos: torch.Tensor, sin: torch.Tensor, extra_tokens: int) -> torch.Tensor:
+        import weakref
+        e = self.entries.get(extra_tokens)
+        if e is not None and e[0]() is cos and e[1]() is sin and e[2] == (cos._version, sin._version):
+            return e[3]
+        table = rope_table_from_cos_sin(cos, sin, extra_tokens=extra_tokens)
+        self.entries[extra_tokens] = (weakref.ref(cos), weakref.ref(sin), (cos._version, sin._version), table)
+        return table
+
+
+_ROTARY_TABLES = _RotaryTableCache()
+
+
 class FusedHunyuanAttnProcessor:
     """``HunyuanVideoAttnProcessor2_0.__call__`` (``teletron/models/hunyuan/model.py:71-170``) with
     the per-head ``attn.norm_q`` / ``attn.norm_k`` and the ``apply_rotary_emb`` that follows them
@@ -283,7 +304,7 @@ class FusedHunyuanAttnProcessor:
             hidden_states = torch.cat([hidden_states, encoder_hidden_states], dim=1)
         heads = attn.heads
         split = lambda t: t.unflatten(2, (heads, -1)).transpose(1, 2)       # [B, S, H*D] -> [B, H, S, D] view
-        table = rope_table_from_cos_sin(image_rotary_emb[0], image_rotary_emb[1], extra_tokens=n_text)
+        table = _ROTARY_TABLES.get(image_rotary_emb[0], image_rotary_emb[1], n_text)   # built once per forward pass
         query = RMSNormRopeHeadsFunction.apply(split(attn.to_q(hidden_states)), attn.norm_q.weight, table, attn.norm_q.eps)
         key = RMSNormRopeHeadsFunction.apply(split(attn.to_k(hidden_states)), attn.norm_k.weight, table, attn.norm_k.eps)
         value = split(attn.to_v(hidden_states))

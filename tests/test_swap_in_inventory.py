@@ -267,3 +267,16 @@ def test_replacement_forwards_keep_the_recorded_signatures():
     calls = spec_of("HunyuanVideoTransformerBlock")["forward_calls"]
     assert {"self.norm1", "self.norm1_context", "self.attn", "self.norm2", "self.norm2_context", "self.ff",
             "self.ff_context", "self.gate"} <= set(calls)
+
+
+def test_rotary_table_cache_follows_the_tensors_it_was_built_from():
+    cos, sin = torch.rand(5, 8), torch.rand(5, 8)
+    cache = S._RotaryTableCache()
+    t1 = cache.get(cos, sin, 2)
+    assert cache.get(cos, sin, 2) is t1                                   # same objects, unmodified: reused
+    assert t1.shape == (7, 4, 2) and torch.equal(t1[5:, :, 0], torch.ones(2, 4)) and not t1[5:, :, 1].any()
+    assert cache.get(cos, sin, 0).shape == (5, 4, 2) and cache.get(cos, sin, 2) is t1   # one entry per text length
+    cos.add_(1.0)
+    t2 = cache.get(cos, sin, 2)
+    assert t2 is not t1 and torch.equal(t2[:5, :, 0], cos[:, 0::2])       # modified in place: rebuilt
+    assert cache.get(cos.clone(), sin, 2) is not t2                       # another tensor object: rebuilt
