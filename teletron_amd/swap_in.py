@@ -34,7 +34,9 @@ ships no code that performs the swap.  This module does it by patching *instance
 
 * HunyuanVideo (``teletron/models/hunyuan/model.py``): ``norm2`` / ``norm2_context`` of
   ``HunyuanVideoTransformerBlock`` with the inline modulation after them (``:615-623,660-669``) go
-  the token way as well; the ``gate(self, x, gate, residual)`` *methods* of both block classes
+  and ``norm`` of the model's ``norm_out`` (diffusers' ``AdaLayerNormContinuous``, ``:759-761,972``, whose
+  ``self.norm(x) * (1 + scale)[:, None, :] + shift[:, None, :]`` is the same inline form) go the token
+  way as well; the ``gate(self, x, gate, residual)`` *methods* of both block classes
   (``:538-539,627-628``) are shadowed by the fused gated residual add; with ``blocks=True`` the
   double-stream block gets a ``forward`` that fuses its first gate with ``norm2`` + modulation
   (:func:`fused_hunyuan_block_forward`) and every attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
@@ -51,10 +53,12 @@ from __future__ import annotations
 
 import os
 import types
+import weakref
 from typing import Callable, Iterable, Optional
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import ops
 from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, RMSNormRopeFunction,
@@ -63,7 +67,8 @@ from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelF
 
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm", "norm2_context")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle",
-                       "HunyuanVideoTransformerBlock")     # hunyuan/model.py:615-623: norm2, norm2_context, inline form
+                       "HunyuanVideoTransformerBlock",     # hunyuan/model.py:615-623: norm2, norm2_context, inline form
+                       "AdaLayerNormContinuous")           # hunyuan/model.py:759-761,972: norm_out (a diffusers class)
 # classes whose ``gate(self, x, gate, residual)`` is a method (hunyuan/model.py:538-539,627-628); context
 # parallelism replaces it by attribute assignment (hunyuan/parallel_model.py:239-244)
 GATE_METHOD_OWNERS = ("HunyuanVideoSingleTransformerBlock", "HunyuanVideoTransformerBlock")
@@ -109,7 +114,7 @@ class DeferredNorm:
 
     def materialize(self) -> torch.Tensor:
         """Plain LayerNorm, for a consumer that is not a modulation."""
-        return torch.nn.functional.layer_norm(self.x, (self.x.shape[-1],), eps=self.eps)
+        return F.layer_norm(self.x, (self.x.shape[-1],), eps=self.eps)
 
     def __getattr__(self, name):
         raise AttributeError(
@@ -170,7 +175,7 @@ class DeferredLayerNorm(nn.Module):
     def forward(self, x: torch.Tensor):
         if x.is_cuda and x.dtype == torch.bfloat16:
             return DeferredNorm(x, self.eps)
-        return torch.nn.functional.layer_norm(x, self.normalized_shape, eps=self.eps)
+        return F.layer_norm(x, self.normalized_shape, eps=self.eps)
 
     def extra_repr(self) -> str:
         return f"{self.normalized_shape}, eps={self.eps}, fused with the following modulation"
@@ -207,8 +212,18 @@ def _fused_gate_forward(self, x, gate, residual):
     return type(self).forward(self, x, gate, residual)
 
 
-def _is_plain_layernorm(m) -> bool:
-    return (isinstance(m, nn.LayerNorm) and not m.elementwise_affine and len(m.normalized_shape) == 1)
+def _plain_layernorm_dim(m) -> Optional[int]:
+    """Width of a LayerNorm over the last dimension without affine parameters, else None:
+    ``nn.LayerNorm(dim, elementwise_affine=False)``, or the module of the same name that diffusers'
+    ``AdaLayerNormContinuous`` holds (a class of its own: ``weight`` and ``bias`` None, the shape in ``dim``)."""
+    if isinstance(m, nn.LayerNorm):
+        return m.normalized_shape[0] if not m.elementwise_affine and len(m.normalized_shape) == 1 else None
+    if (isinstance(m, nn.Module) and type(m).__name__ == "LayerNorm" and hasattr(m, "eps")
+            and getattr(m, "weight", 0) is None and getattr(m, "bias", 0) is None):
+        dim = getattr(m, "dim", None)
+        if isinstance(dim, (tuple, list, torch.Size)) and len(dim) == 1:
+            return int(dim[0])
+    return None
 
 
 BLOCK_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock")   # wan_model.py:212-244, parallel_wan_model.py:12-37
@@ -249,18 +264,24 @@ def fused_self_attention_forward(self, x, freqs):
 class _RotaryTableCache:
     """The fp32 (cos, sin) table of ``rope_table_from_cos_sin`` for the rotary pair a model hands to
     all of its blocks in one forward pass: built on first use, reused while the very same tensor
-    objects (held weakly) are passed again unmodified.  One entry per number of appended text tokens."""
+    objects (held weakly) are passed again unmodified, dropped when they are freed.  One entry per
+    number of appended text tokens."""
 
     def __init__(self):
         self.entries = {}
 
     def get(self, cos: torch.Tensor, sin: torch.Tensor, extra_tokens: int) -> torch.Tensor:
-        import weakref
         e = self.entries.get(extra_tokens)
         if e is not None and e[0]() is cos and e[1]() is sin and e[2] == (cos._version, sin._version):
             return e[3]
         table = rope_table_from_cos_sin(cos, sin, extra_tokens=extra_tokens)
-        self.entries[extra_tokens] = (weakref.ref(cos), weakref.ref(sin), (cos._version, sin._version), table)
+
+        def drop(ref, key=extra_tokens):          # the pair is gone: so is the table built from it
+            held = self.entries.get(key)
+            if held is not None and ref in (held[0], held[1]):
+                del self.entries[key]
+
+        self.entries[extra_tokens] = (weakref.ref(cos, drop), weakref.ref(sin, drop), (cos._version, sin._version), table)
         return table
 
 
@@ -297,7 +318,6 @@ class FusedHunyuanAttnProcessor:
     def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, image_rotary_emb=None):
         if not self._fusable(attn, hidden_states, image_rotary_emb):
             return self.original(attn, hidden_states, encoder_hidden_states, attention_mask, image_rotary_emb)
-        import torch.nn.functional as F
         single_stream = attn.add_q_proj is None and encoder_hidden_states is not None
         n_text = encoder_hidden_states.shape[1] if single_stream else 0
         if single_stream:
@@ -443,8 +463,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
                     counts["modulate"] += 1
             for attr in ADALN_NORM_ATTRS:
                 ln = getattr(module, attr, None)
-                if _is_plain_layernorm(ln):
-                    setattr(module, attr, DeferredLayerNorm(ln.normalized_shape[0], ln.eps))
+                dim = _plain_layernorm_dim(ln)
+                if dim is not None:
+                    setattr(module, attr, DeferredLayerNorm(dim, ln.eps))
                     counts["layernorm"] += 1
     return counts
 

@@ -37,7 +37,7 @@ CLASSES = {
     "wan": ["RMSNorm", "AttentionModule", "SelfAttention", "CrossAttention", "GateModule", "DiTBlock", "Head"],
     "wan_parallel": ["ContextParallelWanDitBlock", "ParallelWanModel"],
     "hunyuan": ["HunyuanVideoAttnProcessor2_0", "FP32LayerNorm", "AdaLayerNormZero", "AdaLayerNormZeroSingle",
-                "HunyuanVideoSingleTransformerBlock", "HunyuanVideoTransformerBlock"],
+                "HunyuanVideoSingleTransformerBlock", "HunyuanVideoTransformerBlock", "HunyuanVideoTransformer3DModel"],
     "hunyuan_parallel": ["HunyuanVideoDoubleAttnProcessor2_0", "HunyuanVideoSingleAttnProcessor2_0",
                          "ParallelHunyuanVideoModel"],
     "cp_layers": ["ContextParallelGateModule", "GateWithGradReduce", "ModulateWithCPGradReduce"],

@@ -4,8 +4,10 @@ HunyuanVideo's blocks in TeleTron (teletron/models/hunyuan/model.py):
   AdaLayerNormZero / ...Single          :425-504  self.modulate(self.norm(x), shift[:, None], scale[:, None])
   HunyuanVideoSingleTransformerBlock    :507-583  method gate(x, gate, residual); text tokens appended
   HunyuanVideoTransformerBlock          :586-681  norm2 / norm2_context + inline modulation; method gate
+  norm_out = AdaLayerNormContinuous     :759-761,972  (a diffusers class) final norm + inline modulation
 The reference needs diffusers (Attention, FeedForward, RMSNorm, apply_rotary_emb), which is not
-installed, so these are written for the tests; `Attention`, `RMSNorm` and `apply_rotary_emb` follow
+installed, so these are written for the tests; `Attention`, `RMSNorm`, `LayerNorm`,
+`AdaLayerNormContinuous` and `apply_rotary_emb` follow
 the published diffusers interfaces the reference relies on (attribute names of the attention
 module, `x * cos + rotate(x) * sin` with tables that hold each value twice in a row).
 """
@@ -125,6 +127,34 @@ class AdaLayerNormZeroSingle(nn.Module):
         return self.modulate(self.norm(x), shift_msa[:, None], scale_msa[:, None]), gate_msa
 
 
+class LayerNorm(nn.Module):
+    """diffusers.models.normalization.LayerNorm: a module of its own (not nn.LayerNorm); without
+    elementwise_affine its weight and bias are None and the normalised shape is kept in `dim`."""
+
+    def __init__(self, dim, eps=1e-5, elementwise_affine=True, bias=True):
+        super().__init__()
+        self.eps, self.dim = eps, torch.Size((dim,))
+        self.weight = nn.Parameter(torch.ones(dim)) if elementwise_affine else None
+        self.bias = nn.Parameter(torch.zeros(dim)) if elementwise_affine and bias else None
+
+    def forward(self, x):
+        return F.layer_norm(x, self.dim, self.weight, self.bias, self.eps)
+
+
+class AdaLayerNormContinuous(nn.Module):
+    """diffusers.models.normalization.AdaLayerNormContinuous with norm_type="layer_norm"."""
+
+    def __init__(self, dim, cond_dim, elementwise_affine=True, eps=1e-5, bias=True):
+        super().__init__()
+        self.silu, self.linear = nn.SiLU(), nn.Linear(cond_dim, 2 * dim, bias=bias)
+        self.norm = LayerNorm(dim, eps, elementwise_affine, bias)
+
+    def forward(self, x, conditioning_embedding):
+        emb = self.linear(self.silu(conditioning_embedding).to(x.dtype))
+        scale, shift = torch.chunk(emb, 2, dim=1)
+        return self.norm(x) * (1 + scale)[:, None, :] + shift[:, None, :]
+
+
 class FeedForward(nn.Sequential):
     def __init__(self, dim, mult=2):
         super().__init__(nn.Linear(dim, mult * dim), nn.GELU(approximate="tanh"), nn.Linear(mult * dim, dim))
@@ -186,13 +216,14 @@ class HunyuanVideoTransformerBlock(nn.Module):
 
 
 class TwoStreamModel(nn.Module):
-    """One double-stream block followed by one single-stream block, as the transformer chains them
-    (hunyuan/model.py:936-969)."""
+    """One double-stream block followed by one single-stream block and the output normalisation of
+    the latent stream, as the transformer chains them (hunyuan/model.py:759-761,936-972)."""
 
     def __init__(self, heads, head_dim):
         super().__init__()
         self.transformer_blocks = nn.ModuleList([HunyuanVideoTransformerBlock(heads, head_dim)])
         self.single_transformer_blocks = nn.ModuleList([HunyuanVideoSingleTransformerBlock(heads, head_dim)])
+        self.norm_out = AdaLayerNormContinuous(heads * head_dim, heads * head_dim, elementwise_affine=False, eps=1e-6)
 
     def forward(self, hidden_states, encoder_hidden_states, temb, cos, sin):
         rotary = (cos, sin)
@@ -200,4 +231,4 @@ class TwoStreamModel(nn.Module):
             hidden_states, encoder_hidden_states = blk(hidden_states, encoder_hidden_states, temb, None, rotary)
         for blk in self.single_transformer_blocks:
             hidden_states, encoder_hidden_states = blk(hidden_states, encoder_hidden_states, temb, None, rotary)
-        return torch.cat([hidden_states, encoder_hidden_states], dim=1)
+        return torch.cat([self.norm_out(hidden_states, temb), encoder_hidden_states], dim=1)

@@ -50,12 +50,13 @@ def test_hunyuan_swap_in_matches_eager_model(head_dim):
     keys_before = list(wrapped.state_dict().keys())
     out_e, gin_e, gp_e = run(wrapped, inputs, dy)
     counts = S.swap_in(wrapped, blocks=True)
-    # LayerNorms: norm1.norm, norm1_context.norm, norm2, norm2_context, single norm.norm; modulate attributes of
+    # LayerNorms: norm1.norm, norm1_context.norm, norm2, norm2_context, single norm.norm, norm_out.norm; modulate attributes of
     # the three AdaLayerNormZero[Single]; the gate method of each block; q/k (+ added q/k) RMSNorms; two processors
-    assert counts == {"rmsnorm": 6, "layernorm": 5, "modulate": 3, "gate": 2, "block": 1, "attention": 0,
+    assert counts == {"rmsnorm": 6, "layernorm": 6, "modulate": 3, "gate": 2, "block": 1, "attention": 0,
                       "processor": 2}, counts
     dbl, sgl = model.transformer_blocks[0], model.single_transformer_blocks[0]
     assert isinstance(dbl.norm2, S.DeferredLayerNorm) and isinstance(dbl.norm2_context, S.DeferredLayerNorm)
+    assert isinstance(model.norm_out.norm, S.DeferredLayerNorm)
     assert isinstance(dbl.attn.processor, S.FusedHunyuanAttnProcessor) and isinstance(sgl.attn.processor, S.FusedHunyuanAttnProcessor)
     assert "gate" in dbl.__dict__ and "gate" in sgl.__dict__ and "forward" in dbl.__dict__
     assert list(wrapped.state_dict().keys()) == keys_before
@@ -112,7 +113,7 @@ def test_context_parallel_gate_assignment(monkeypatch):
     wrapped = WithRotary(model, rotary)
     out_e, _, _ = run(wrapped, inputs, dy)
     counts = S.swap_in(wrapped)
-    assert counts["gate"] == 2 and counts["modulate"] == 3 and counts["layernorm"] == 5, counts
+    assert counts["gate"] == 2 and counts["modulate"] == 3 and counts["layernorm"] == 6, counts
     out_f, _, _ = run(wrapped, inputs, dy)
     assert rel(out_f, out_e) < 5e-3
 
@@ -120,7 +121,7 @@ def test_context_parallel_gate_assignment(monkeypatch):
     monkeypatch.setattr(S, "_several_ranks", lambda: True)
     counts = S.swap_in(WithRotary(model, rotary))
     # gates stay; the two owners whose modulate is the CP callable keep their LayerNorm as well;
-    # norm1_context (plain modulate) and norm2 / norm2_context (inline, row-local) are swapped
-    assert counts["gate"] == 0 and counts["modulate"] == 1 and counts["layernorm"] == 3, counts
+    # norm1_context (plain modulate) and norm2 / norm2_context / norm_out (inline, row-local) are swapped
+    assert counts["gate"] == 0 and counts["modulate"] == 1 and counts["layernorm"] == 4, counts
     assert isinstance(model.transformer_blocks[0].norm1.norm, nn.LayerNorm)
     assert not hasattr(model.transformer_blocks[0].gate, "__wrapped__")

@@ -62,9 +62,25 @@ def make_attention(kwargs):
     return m
 
 
+def make_ada_layer_norm_continuous(kwargs):
+    """diffusers' AdaLayerNormContinuous is not part of the reference sources either: built with the
+    recorded constructor keywords in its published form, a `norm` child of diffusers' own LayerNorm
+    class (weight = bias = None without elementwise_affine, the normalised shape in `dim`)."""
+    ln = type("LayerNorm", (Shell,), {})()
+    ln.eps, ln.dim = kwargs.get("eps", 1e-5), torch.Size((DIM,))
+    affine = kwargs.get("elementwise_affine", True)
+    ln.weight = nn.Parameter(torch.ones(DIM)) if affine else None
+    ln.bias = nn.Parameter(torch.zeros(DIM)) if affine else None
+    m = type("AdaLayerNormContinuous", (Shell,), {})()
+    m.silu, m.linear, m.norm = nn.Identity(), nn.Identity(), ln
+    return m
+
+
 def build(name, kwargs=None):
     """An instance with the recorded class name, children and methods."""
     kwargs = kwargs or {}
+    if name == "AdaLayerNormContinuous":
+        return make_ada_layer_norm_continuous(kwargs)
     if name == "LayerNorm":
         return nn.LayerNorm(DIM, eps=1e-6, elementwise_affine=kwargs.get("elementwise_affine", True))
     if name == "RMSNorm":
@@ -111,6 +127,8 @@ def expected_sites(root):
             want[path] = "rmsnorm"
         if name in ("GateModule", "ContextParallelGateModule"):
             want[path] = "gate-module"
+        if name == "AdaLayerNormContinuous" and m.norm.weight is None:
+            want[path + ".norm"] = "adaln"
         if spec is None:
             continue
         uses = forward_uses(spec)
@@ -205,6 +223,24 @@ def test_swap_in_patches_every_recorded_site_and_nothing_else(blocks):
     assert counts["layernorm"] == 8 and counts["gate"] == 4 and counts["rmsnorm"] == 11, counts
 
 
+def test_output_norm_of_the_hunyuan_model_is_a_recorded_site():
+    """HunyuanVideoTransformer3DModel.norm_out: AdaLayerNormContinuous(elementwise_affine=False, eps=1e-6),
+    applied to the latent stream just before proj_out (hunyuan/model.py:759-761,972)."""
+    spec = spec_of("HunyuanVideoTransformer3DModel")
+    (child,) = [c for c in spec["children"] if c["attr"] == "norm_out"]
+    assert child["class"] == "AdaLayerNormContinuous" and child["kwargs"] == {"elementwise_affine": False, "eps": 1e-6}
+    assert {"attr": "norm_out", "consumer": "call:self.proj_out"} in spec["forward_uses_of_self_attributes"]
+    root = nn.Module()
+    root.norm_out = build(child["class"], child["kwargs"])
+    root.affine = build(child["class"], {"elementwise_affine": True})      # with parameters: not an AdaLN site
+    want = expected_sites(root)
+    assert want == {"norm_out.norm": "adaln"}
+    before = dict(root.named_modules())
+    counts = S.swap_in(root, blocks=True)
+    assert patched_sites(root, before) == want and counts["layernorm"] == 1
+    assert root.norm_out.norm.eps == 1e-6 and root.norm_out.norm.normalized_shape == (DIM,)
+
+
 def test_context_parallel_assignments_are_recognised(monkeypatch):
     """What ParallelHunyuanVideoModel.__init__ assigns onto its blocks and what the context-parallel
     Wan block calls are the names swap_in knows; with several ranks they are left alone."""
@@ -280,3 +316,6 @@ def test_rotary_table_cache_follows_the_tensors_it_was_built_from():
     t2 = cache.get(cos, sin, 2)
     assert t2 is not t1 and torch.equal(t2[:5, :, 0], cos[:, 0::2])       # modified in place: rebuilt
     assert cache.get(cos.clone(), sin, 2) is not t2                       # another tensor object: rebuilt
+    assert 2 not in cache.entries and 0 in cache.entries                  # ... and dropped with that object
+    del cos, sin
+    assert not cache.entries
