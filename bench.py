@@ -451,7 +451,7 @@ def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3
             "relative_output_difference": diff, "swapped": counts}
 
 
-def function_path(w, cabi_ms, iters=10):
+def function_path(w, cabi_ms, iters=50):
     """The path model code calls: AdaLNModelFunction / RMSNormModelFunction apply + backward on
     tensors of the workload's shape, parameters as the model passes them ([B, 1, C] modulation,
     [C] weight), two alternating input sets.  Wall milliseconds per forward+backward and the

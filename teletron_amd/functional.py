@@ -44,11 +44,13 @@ class AdaLNModelFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         x, scale_c = ctx.saved_tensors
-        dx, dscale, dshift = ops.adaln_backward(grad_output.contiguous(), x, scale_c, ctx.eps)
+        dx, grads = ops.adaln_backward_packed(grad_output.contiguous(), x, scale_c, ctx.eps)
         (sc_shape, sc_dtype), (sh_shape, sh_dtype) = ctx.scale_meta, ctx.shift_meta
+        if sc_dtype == sh_dtype:
+            grads = grads.to(sc_dtype)          # both parameter gradients in one cast
         dx = dx if ctx.needs_input_grad[0] else None
-        dscale = dscale.to(sc_dtype).reshape(sc_shape) if ctx.needs_input_grad[1] else None
-        dshift = dshift.to(sh_dtype).reshape(sh_shape) if ctx.needs_input_grad[2] else None
+        dscale = grads[0].to(sc_dtype).reshape(sc_shape) if ctx.needs_input_grad[1] else None
+        dshift = grads[1].to(sh_dtype).reshape(sh_shape) if ctx.needs_input_grad[2] else None
         return dx, dscale, dshift, None, None
 
 

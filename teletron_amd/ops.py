@@ -128,8 +128,9 @@ def adaln_forward(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps
     return (y, mean, rstd) if return_stats else y
 
 
-def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: float):
-    """Returns (dx bf16 like x, dscale fp32 [n_batches, C], dshift fp32 [n_batches, C])."""
+def adaln_backward_packed(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: float):
+    """Returns (dx bf16 like x, grads fp32 [2, n_batches, C]) with grads[0] = dscale, grads[1] = dshift:
+    one tensor, so that a caller casting both to the parameters' dtype needs one launch for it."""
     cols = x.shape[-1]
     x = _check_act("x", x, cols)
     dy = _check_act("dy", dy, cols)
@@ -138,16 +139,20 @@ def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: 
     rows, nb, rpb = _batches(x, scale, cols)
     dx = torch.empty_like(x)
     if rows == 0:
-        z = torch.zeros(nb, cols, dtype=torch.float32, device=x.device)
-        return dx, z, z.clone()
-    dscale = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
-    dshift = torch.empty(nb, cols, dtype=torch.float32, device=x.device)
+        return dx, torch.zeros(2, nb, cols, dtype=torch.float32, device=x.device)
+    grads = torch.empty(2, nb, cols, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         ws = _workspace(cabi.load().tt_adaln_backward_workspace_bytes(rows, cols, rpb), rows, x, dy, dx, scale)
-        cabi.call("tt_adaln_backward", dx.data_ptr(), dscale.data_ptr(), dshift.data_ptr(),
+        cabi.call("tt_adaln_backward", dx.data_ptr(), grads[0].data_ptr(), grads[1].data_ptr(),
                   dy.data_ptr(), x.data_ptr(), scale.data_ptr(), ws.data_ptr(), ws.numel(),
                   rows, cols, rpb, float(eps), _stream(x))
-    return dx, dscale, dshift
+    return dx, grads
+
+
+def adaln_backward(dy: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, eps: float):
+    """Returns (dx bf16 like x, dscale fp32 [n_batches, C], dshift fp32 [n_batches, C])."""
+    dx, grads = adaln_backward_packed(dy, x, scale, eps)
+    return dx, grads[0], grads[1]
 
 
 def rmsnorm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float, return_stats: bool = False):
