@@ -1,4 +1,4 @@
-"""Writes tests/golden/wan_block_vectors.npz: inputs and float32 CPU results (output, input
+"""Writes tests/golden/model/wan_block_vectors.npz: inputs and float32 CPU results (output, input
 gradients, parameter gradients) of the reference's REAL DiTBlock / Head classes on the case defined
 in tests/wan_standins.py (two blocks + head, 2 x 40 tokens of width 512, per-sample modulation).
 
@@ -47,7 +47,7 @@ def main():
             arrays["grad_right/" + n], arrays["grad_left/" + n] = W.matrix_summary(g)
         else:
             arrays["grad/" + n] = g
-    path = os.path.join(HERE, "wan_block_vectors.npz")
+    path = os.path.join(HERE, "model", "wan_block_vectors.npz")
     np.savez_compressed(path, **arrays)
     print("wrote", path, os.path.getsize(path), "bytes;", len(names), "parameters; |out| =", float(out.abs().mean()))
 

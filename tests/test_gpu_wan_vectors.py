@@ -1,5 +1,5 @@
 """The fused kernels, swapped into the Wan stand-ins, against the numbers of the reference's REAL
-DiTBlock / Head classes (tests/golden/wan_block_vectors.npz: float32 CPU results of
+DiTBlock / Head classes (tests/golden/model/wan_block_vectors.npz: float32 CPU results of
 teletron/models/wan/wan_model.py:212-278 on the case of tests/wan_standins.py; the stand-ins are
 pinned to the same file on the CPU by tests/test_wan_vectors.py).  The model runs in bf16 on the GPU,
 eager and after swap_in(blocks=True); both are compared with the float32 truth, and the fused model

@@ -1,5 +1,5 @@
 """The Wan stand-ins of tests/wan_standins.py against the numbers of the reference's real classes
-(tests/golden/wan_block_vectors.npz, written by tests/golden/make_wan_block_vectors.py): same
+(tests/golden/model/wan_block_vectors.npz, written by tests/golden/make_wan_block_vectors.py): same
 parameters, same inputs, float32 on the CPU.  Pins the stand-ins that the swap-in tests rely on to
 teletron/models/wan/wan_model.py:77-278 numerically, and their state-dict keys to the real ones."""
 import os
@@ -9,7 +9,7 @@ import torch
 
 import wan_standins as W
 
-GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "wan_block_vectors.npz"))
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "model", "wan_block_vectors.npz"))
 
 
 def close(got, want, rtol=2e-4):

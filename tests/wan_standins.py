@@ -9,7 +9,7 @@ reference's numbers (teletron/models/wan/wan_model.py):
   DiTBlock                 :212-244
   Head                     :266-278
 Same class names, attribute names, parameter names and call order, so a state dict of the real
-classes loads.  tests/golden/wan_block_vectors.npz holds inputs and fp32 results of the REAL classes
+classes loads.  tests/golden/model/wan_block_vectors.npz holds inputs and fp32 results of the REAL classes
 (written by tests/golden/make_wan_block_vectors.py in the build container, where the reference can
 be loaded); tests/test_wan_vectors.py checks these stand-ins against it on the CPU, and
 tests/test_gpu_wan_vectors.py the swapped-in fused kernels.
