@@ -27,7 +27,10 @@ build is the *formula evaluated without intermediate rounding*, which is what is
 written here.  Every function below is pinned in ``tests/test_oracle.py`` against
 torch's library routines (``F.layer_norm`` / ``F.rms_norm`` + autograd), against
 central finite differences of a pure-Python scalar implementation, and against
-closed-form special cases.  No function here is "parity unpinned".
+closed-form special cases; ``tests/test_wan_vectors.py`` additionally holds the
+AdaLN and RMSNorm functions against what the reference's own ``RMSNorm`` class and
+``modulate(LayerNorm(x))`` computed in float32 on seeded inputs
+(``tests/golden/model/wan_op_vectors.npz``).  No function here is "parity unpinned".
 
 Shapes: ``x``, ``dy`` are ``[B, S, C]`` (any leading dims are flattened by the
 callers); ``scale`` / ``shift`` are ``[B, C]`` (or ``[1, C]`` broadcast over B);

@@ -203,3 +203,29 @@ def matrix_summary(g):
     rs = np.random.RandomState(7)
     u, v = rs.standard_normal(g.shape[1]), rs.standard_normal(g.shape[0])
     return g @ u, v @ g
+
+
+# ------------------------------------------------------------------ the op-level cases of wan_op_vectors.npz
+OP_CASES = {
+    "rmsnorm_1536": dict(op="rmsnorm", shape=(2, 3, 1536), cols=1536, eps=1e-6, seed=31),
+    "rmsnorm_128": dict(op="rmsnorm", shape=(2, 3, 4, 128), cols=128, eps=1e-6, seed=32),      # one head per row
+    "rmsnorm_1000": dict(op="rmsnorm", shape=(1, 5, 1000), cols=1000, eps=1e-5, seed=33),      # ragged width
+    "adaln_1536": dict(op="adaln", shape=(2, 3, 1536), cols=1536, eps=1e-6, seed=34),
+    "adaln_5120": dict(op="adaln", shape=(1, 2, 5120), cols=5120, eps=1e-6, seed=35),
+    "adaln_offset": dict(op="adaln", shape=(3, 2, 512), cols=512, eps=1e-6, seed=36, offset=30.0),   # |mean| >> std
+}
+
+
+def op_case_inputs(name):
+    """float32 inputs of an op case; the values are exactly representable in bfloat16, so the float32
+    and the bfloat16 runs of the reference see the same numbers."""
+    case = OP_CASES[name]
+    rs = np.random.RandomState(case["seed"])
+    bf = lambda a: torch.from_numpy(a.astype(np.float32)).bfloat16().float()
+    shape, c = case["shape"], case["cols"]
+    out = {"x": bf(case.get("offset", 0.0) + rs.standard_normal(shape)), "dy": bf(rs.standard_normal(shape))}
+    if case["op"] == "rmsnorm":
+        out["weight"] = bf(1.0 + 0.1 * rs.standard_normal(c))
+    else:
+        out["t_mod"] = bf(0.3 * rs.standard_normal((shape[0], 6, c)))
+    return out
