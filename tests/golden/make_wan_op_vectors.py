@@ -1,6 +1,7 @@
 """Writes tests/golden/model/wan_op_vectors.npz: the two ops of the hot path computed by the
-reference's OWN code (teletron/models/wan/wan_model.py: class RMSNorm :113-124; modulate :77-78 applied
-to nn.LayerNorm(dim, eps, elementwise_affine=False) as DiTBlock does, :222-223,236), forward and
+reference's OWN code (teletron/models/wan/wan_model.py: class RMSNorm :113-124, alone and followed by
+rope_apply :105-110 as in SelfAttention.forward; modulate :77-78 applied to
+nn.LayerNorm(dim, eps, elementwise_affine=False) as DiTBlock does, :222-223,236), forward and
 autograd backward, on small seeded inputs: in float32 (the exact formula) and in bfloat16 (what the
 model really computes, with its own cast order).
 
@@ -34,12 +35,14 @@ def main():
             ins = W.op_case_inputs(name)
             x = ins["x"].to(dtype).requires_grad_(True)
             dy = ins["dy"].to(dtype)
-            if case["op"] == "rmsnorm":
+            if case["op"] in ("rmsnorm", "rmsnorm_rope"):
                 m = ref.RMSNorm(case["cols"], eps=case["eps"])
                 with torch.no_grad():
                     m.weight.copy_(ins["weight"])
                 m = m.to(dtype)
                 y = m(x)
+                if case["op"] == "rmsnorm_rope":         # as SelfAttention.forward does with q and k (:154-158)
+                    y = ref.rope_apply(y, W.freqs_from_angles(ins["angles"]), case["heads"])
                 y.backward(dy)
                 grads = {"dweight": m.weight.grad}
             else:

@@ -73,7 +73,7 @@ def test_fused_ops_against_the_reference_codes_numbers(name):
     within the stated tolerance of the float32 results (bf16 outputs 1e-2 + 8e-3 |ref|; parameter
     gradients 1e-3 |ref| + 1e-4 sqrt(rows)), and within three bf16 steps of the reference's bf16 run,
     which rounds after every operation where the kernel rounds once."""
-    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction
+    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction, RMSNormRopeFunction
     from test_wan_vectors import op_reference
     case, ins = W.OP_CASES[name], W.op_case_inputs(name)
     f32, b16 = op_reference(name, "f32"), op_reference(name, "bf16")
@@ -83,6 +83,12 @@ def test_fused_ops_against_the_reference_codes_numbers(name):
         w = ins["weight"].bfloat16().to(DEV).requires_grad_(True)
         RMSNormModelFunction.apply(x, w, case["eps"], case["cols"]).backward(dy)
         y = RMSNormModelFunction.apply(x.detach(), w.detach(), case["eps"], case["cols"])
+        got = {"y": y, "dx": x.grad, "dweight": w.grad}
+    elif case["op"] == "rmsnorm_rope":
+        w = ins["weight"].bfloat16().to(DEV).requires_grad_(True)
+        freqs = W.freqs_from_angles(ins["angles"]).to(DEV)                   # complex128 [S, 1, D/2], as the model passes it
+        RMSNormRopeFunction.apply(x, w, freqs, case["eps"], case["heads"]).backward(dy)
+        y = RMSNormRopeFunction.apply(x.detach(), w.detach(), freqs, case["eps"], case["heads"])
         got = {"y": y, "dx": x.grad, "dweight": w.grad}
     else:
         t_mod = ins["t_mod"].bfloat16().to(DEV).requires_grad_(True)

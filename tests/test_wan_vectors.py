@@ -77,6 +77,12 @@ def oracle_results(name):
         y = O.rmsnorm_forward(ins["x"], ins["weight"], case["eps"])[0]
         dx, dw = O.rmsnorm_backward(ins["dy"], ins["x"], ins["weight"], case["eps"])
         return {"y": y, "dx": dx, "dweight": dw}
+    if case["op"] == "rmsnorm_rope":
+        d = case["cols"] // case["heads"]
+        table = torch.view_as_real(W.freqs_from_angles(ins["angles"])).reshape(-1, d // 2, 2)     # [S, D/2, (cos, sin)]
+        y = O.rmsnorm_rope_forward(ins["x"], ins["weight"], table, case["eps"], d)[0]
+        dx, dw = O.rmsnorm_rope_backward(ins["dy"], ins["x"], ins["weight"], table, case["eps"], d)
+        return {"y": y, "dx": dx, "dweight": dw}
     nb = case["shape"][0]
     shift, scale = ins["t_mod"][:, 0], ins["t_mod"][:, 1]
     y = O.adaln_forward(ins["x"], scale, shift, case["eps"], nb)[0]
@@ -108,6 +114,8 @@ def test_eager_restatement_is_the_reference_code_in_bfloat16():
         if case["op"] == "rmsnorm":
             y, dx, dw = E.eager_rmsnorm_fwd_bwd(x, ins["weight"].bfloat16(), dy, case["eps"])
             got = {"y": y, "dx": dx, "dweight": dw}
+        elif case["op"] == "rmsnorm_rope":
+            continue        # the CPU baseline has no rotary leg
         else:
             t = ins["t_mod"].bfloat16()
             y, dx, dscale, dshift = E.eager_adaln_fwd_bwd(x, t[:, 1:2], t[:, 0:1], dy, case["eps"])

@@ -213,6 +213,7 @@ OP_CASES = {
     "adaln_1536": dict(op="adaln", shape=(2, 3, 1536), cols=1536, eps=1e-6, seed=34),
     "adaln_5120": dict(op="adaln", shape=(1, 2, 5120), cols=5120, eps=1e-6, seed=35),
     "adaln_offset": dict(op="adaln", shape=(3, 2, 512), cols=512, eps=1e-6, seed=36, offset=30.0),   # |mean| >> std
+    "rmsnorm_rope_512": dict(op="rmsnorm_rope", shape=(2, 6, 512), cols=512, heads=4, eps=1e-6, seed=37),   # norm_q + rope_apply
 }
 
 
@@ -224,8 +225,10 @@ def op_case_inputs(name):
     bf = lambda a: torch.from_numpy(a.astype(np.float32)).bfloat16().float()
     shape, c = case["shape"], case["cols"]
     out = {"x": bf(case.get("offset", 0.0) + rs.standard_normal(shape)), "dy": bf(rs.standard_normal(shape))}
-    if case["op"] == "rmsnorm":
+    if case["op"] in ("rmsnorm", "rmsnorm_rope"):
         out["weight"] = bf(1.0 + 0.1 * rs.standard_normal(c))
     else:
         out["t_mod"] = bf(0.3 * rs.standard_normal((shape[0], 6, c)))
+    if case["op"] == "rmsnorm_rope":       # one rotation angle per token and pair, float64 as precompute_freqs_cis
+        out["angles"] = torch.from_numpy(3.0 * rs.standard_normal((shape[-2], 1, c // case["heads"] // 2)))
     return out
