@@ -451,6 +451,61 @@ def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3
             "relative_output_difference": diff, "swapped": counts}
 
 
+def hunyuan_block_demo(n_img=16384, n_txt=256, n_single=3, heads=24, head_dim=128, iters=4):
+    """Whole-block view for HunyuanVideo (--block-demo): `n_single` single-stream blocks in a row, built
+    from the stand-ins the swap-in tests use (tests/hunyuan_standins.py: the call pattern of
+    teletron/models/hunyuan/model.py:64-170,472-583 around nn.Linear and torch SDPA), forward +
+    backward in eager PyTorch, after swap_in() and after swap_in(blocks=True) (fused per-head norm +
+    rotary embedding in the processor, token sequence no longer copied at every re-join)."""
+    import torch
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
+    import hunyuan_standins as H
+    from teletron_amd import swap_in as S
+    dev, bf, dim = "cuda:0", torch.bfloat16, heads * head_dim
+
+    def build():
+        torch.manual_seed(0)
+        return torch.nn.ModuleList([H.HunyuanVideoSingleTransformerBlock(heads, head_dim, mlp_ratio=4)
+                                    for _ in range(n_single)]).to(dev).to(bf)
+
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: torch.randn(*shape, device=dev, generator=g)
+    h, e, temb = rnd(1, n_img, dim).to(bf), rnd(1, n_txt, dim).to(bf), rnd(1, dim).to(bf)
+    ang = 3.0 * rnd(n_img, head_dim // 2)
+    rotary = (ang.cos().repeat_interleave(2, 1), ang.sin().repeat_interleave(2, 1))
+    dy = rnd(1, n_img + n_txt, dim).to(bf)
+
+    def step(m, hh, ee):
+        for blk in m:
+            hh, ee = blk(hh, ee, temb, None, rotary)
+        out = torch.cat([hh, ee], 1)
+        out.backward(dy)
+        return out.detach()
+
+    def timed(m):
+        hh, ee = h.clone().requires_grad_(True), e.clone().requires_grad_(True)
+        for i in range(2 + iters):
+            if i == 2:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            out = step(m, hh, ee)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e3, out
+
+    eager_ms, out_e = timed(build())
+    m = build()
+    S.swap_in(m)
+    swapped_ms, _ = timed(m)
+    m = build()
+    counts = S.swap_in(m, blocks=True)
+    blocks_ms, out_f = timed(m)
+    diff = float((out_f.double() - out_e.double()).norm() / out_e.double().norm())
+    return {"block": f"{n_single} HunyuanVideoSingleTransformerBlock stand-ins, dim {dim}, {heads} heads, "
+                     f"{n_img} latent + {n_txt} text tokens, bf16",
+            "eager_ms": round(eager_ms, 2), "swap_in_ms": round(swapped_ms, 2), "swap_in_blocks_ms": round(blocks_ms, 2),
+            "speedup": round(eager_ms / blocks_ms, 3), "relative_output_difference": diff, "swapped": counts}
+
+
 def function_path(w, cabi_ms, iters=50):
     """The path model code calls: AdaLNModelFunction / RMSNormModelFunction apply + backward on
     tensors of the workload's shape, parameters as the model passes them ([B, 1, C] modulation,
@@ -626,7 +681,7 @@ def main():
     if also:
         out["also"] = also
     if args.block_demo:
-        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824)]
+        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824), hunyuan_block_demo()]
     if args.calibrate_copy:
         src = torch.empty(w.elements, dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
         dst = torch.empty_like(src)

@@ -39,7 +39,8 @@ ships no code that performs the swap.  This module does it by patching *instance
   way as well; the ``gate(self, x, gate, residual)`` *methods* of both block classes
   (``:538-539,627-628``) are shadowed by the fused gated residual add; with ``blocks=True`` the
   double-stream block gets a ``forward`` that fuses its first gate with ``norm2`` + modulation
-  (:func:`fused_hunyuan_block_forward`) and every attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
+  (:func:`fused_hunyuan_block_forward`), the single-stream block one that stops copying the token
+  sequence each time it re-joins latent and text tokens (:func:`fused_hunyuan_single_block_forward`), and every attention module driven by ``HunyuanVideoAttnProcessor2_0`` (``:64-170``) gets
   :class:`FusedHunyuanAttnProcessor`, which runs ``norm_q`` / ``norm_k`` and the rotary embedding
   after them as one kernel per tensor (text tokens appended to the latent ones take no rotation).
 
@@ -288,6 +289,31 @@ class _RotaryTableCache:
 _ROTARY_TABLES = _RotaryTableCache()
 
 
+def split_tokens(t: torch.Tensor, n_text: int):
+    """``t[:, :-n_text], t[:, -n_text:]`` (latent tokens, appended text tokens), each half remembering
+    the tensor it was cut from so that :func:`join_tokens` can hand that tensor back."""
+    a, b = t[:, :-n_text, :], t[:, -n_text:, :]
+    a._tt_whole = b._tt_whole = t
+    return a, b
+
+
+def join_tokens(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``torch.cat([a, b], dim=1)``; when ``a`` and ``b`` are the two halves that :func:`split_tokens`
+    cut from one tensor, still in place, that tensor itself: no copy in forward and, in backward, no
+    zero-filled gradient per half with an addition after them.  HunyuanVideo's single-stream block
+    splits and re-joins its tokens three times per block (``hunyuan/model.py:549-582`` with the
+    processor's ``:79-81,143-146``); between the fused block forwards and the fused processor of this
+    module the halves carry the hint, anything else is concatenated as before."""
+    t = getattr(a, "_tt_whole", None)
+    if (t is not None and t is getattr(b, "_tt_whole", None) and t.dim() == 3 and a.dim() == 3 and b.dim() == 3
+            and a.shape[1] + b.shape[1] == t.shape[1] and a.shape[0] == b.shape[0] == t.shape[0]
+            and a.shape[2] == b.shape[2] == t.shape[2] and a.stride() == t.stride() == b.stride()
+            and a.data_ptr() == t.data_ptr() and b.data_ptr() == t.data_ptr() + a.shape[1] * t.stride(1) * t.element_size()
+            and a.requires_grad == t.requires_grad == b.requires_grad):
+        return t
+    return torch.cat([a, b], dim=1)
+
+
 class FusedHunyuanAttnProcessor:
     """``HunyuanVideoAttnProcessor2_0.__call__`` (``teletron/models/hunyuan/model.py:71-170``) with
     the per-head ``attn.norm_q`` / ``attn.norm_k`` and the ``apply_rotary_emb`` that follows them
@@ -321,7 +347,7 @@ class FusedHunyuanAttnProcessor:
         single_stream = attn.add_q_proj is None and encoder_hidden_states is not None
         n_text = encoder_hidden_states.shape[1] if single_stream else 0
         if single_stream:
-            hidden_states = torch.cat([hidden_states, encoder_hidden_states], dim=1)
+            hidden_states = join_tokens(hidden_states, encoder_hidden_states)
         heads = attn.heads
         split = lambda t: t.unflatten(2, (heads, -1)).transpose(1, 2)       # [B, S, H*D] -> [B, H, S, D] view
         table = _ROTARY_TABLES.get(image_rotary_emb[0], image_rotary_emb[1], n_text)   # built once per forward pass
@@ -345,8 +371,7 @@ class FusedHunyuanAttnProcessor:
                                                        is_causal=False)
         hidden_states = hidden_states.transpose(1, 2).flatten(2, 3).to(query.dtype)
         if encoder_hidden_states is not None:
-            n_enc = encoder_hidden_states.shape[1]
-            hidden_states, encoder_hidden_states = hidden_states[:, :-n_enc], hidden_states[:, -n_enc:]
+            hidden_states, encoder_hidden_states = split_tokens(hidden_states, encoder_hidden_states.shape[1])
             if getattr(attn, "to_out", None) is not None:
                 hidden_states = attn.to_out[1](attn.to_out[0](hidden_states))
             if getattr(attn, "to_add_out", None) is not None:
@@ -380,6 +405,32 @@ def fused_hunyuan_block_forward(self, hidden_states, encoder_hidden_states, temb
     hidden_states = self.gate(hidden_states, gate_mlp.unsqueeze(1), ff_output)
     encoder_hidden_states = encoder_hidden_states + c_gate_mlp.unsqueeze(1) * context_ff_output
     return hidden_states, encoder_hidden_states
+
+
+def fused_hunyuan_single_block_forward(self, hidden_states, encoder_hidden_states, temb, attention_mask=None,
+                                       image_rotary_emb=None):
+    """``HunyuanVideoSingleTransformerBlock.forward`` (``hunyuan/model.py:541-583``) in the reference's
+    order with its own, possibly swapped, sub-modules; the three places where it concatenates the
+    latent and the text tokens that it (or the block before it, or the attention processor) had just
+    cut apart go through :func:`join_tokens`, which takes the uncut tensor instead of a copy."""
+    n_text = encoder_hidden_states.shape[1]
+    hidden_states = join_tokens(hidden_states, encoder_hidden_states)
+    residual = hidden_states
+    norm_hidden_states, gate = self.norm(hidden_states, emb=temb)
+    mlp_hidden_states = self.act_mlp(self.proj_mlp(norm_hidden_states))
+    norm_hidden_states, norm_encoder_hidden_states = split_tokens(norm_hidden_states, n_text)
+    attn_output, context_attn_output = self.attn(hidden_states=norm_hidden_states,
+                                                 encoder_hidden_states=norm_encoder_hidden_states,
+                                                 attention_mask=attention_mask, image_rotary_emb=image_rotary_emb)
+    attn_output = join_tokens(attn_output, context_attn_output)
+    hidden_states = self.proj_out(torch.cat([attn_output, mlp_hidden_states], dim=2))
+    hidden_states = self.gate(residual, gate.unsqueeze(1), hidden_states)
+    return split_tokens(hidden_states, n_text)
+
+
+def _is_hunyuan_single_block(m: nn.Module) -> bool:
+    return (type(m).__name__ == "HunyuanVideoSingleTransformerBlock"
+            and all(hasattr(m, a) for a in ("norm", "attn", "proj_mlp", "act_mlp", "proj_out", "gate")))
 
 
 def _is_hunyuan_double_block(m: nn.Module) -> bool:
@@ -430,6 +481,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
             counts["block"] += 1
         if blocks and adaln and gate and _is_hunyuan_double_block(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_hunyuan_block_forward, module)
+            counts["block"] += 1
+        if blocks and _is_hunyuan_single_block(module) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(fused_hunyuan_single_block_forward, module)
             counts["block"] += 1
         if blocks and rmsnorm and _is_self_attention(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_self_attention_forward, module)

@@ -219,10 +219,11 @@ class TwoStreamModel(nn.Module):
     """One double-stream block followed by one single-stream block and the output normalisation of
     the latent stream, as the transformer chains them (hunyuan/model.py:759-761,936-972)."""
 
-    def __init__(self, heads, head_dim):
+    def __init__(self, heads, head_dim, n_single=1):
         super().__init__()
         self.transformer_blocks = nn.ModuleList([HunyuanVideoTransformerBlock(heads, head_dim)])
-        self.single_transformer_blocks = nn.ModuleList([HunyuanVideoSingleTransformerBlock(heads, head_dim)])
+        self.single_transformer_blocks = nn.ModuleList([HunyuanVideoSingleTransformerBlock(heads, head_dim)
+                                                        for _ in range(n_single)])
         self.norm_out = AdaLayerNormContinuous(heads * head_dim, heads * head_dim, elementwise_affine=False, eps=1e-6)
 
     def forward(self, hidden_states, encoder_hidden_states, temb, cos, sin):

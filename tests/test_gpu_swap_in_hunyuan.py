@@ -15,10 +15,10 @@ from test_gpu_swap_in import rel, run
 pytestmark = pytest.mark.gpu
 
 
-def make_model_and_inputs(seed=0, heads=4, head_dim=64, bsz=2, n_img=96, n_txt=16):
+def make_model_and_inputs(seed=0, heads=4, head_dim=64, bsz=2, n_img=96, n_txt=16, n_single=1):
     torch.manual_seed(seed)
     dim = heads * head_dim
-    model = H.TwoStreamModel(heads, head_dim).to(DEV).to(torch.bfloat16)
+    model = H.TwoStreamModel(heads, head_dim, n_single).to(DEV).to(torch.bfloat16)
     with torch.no_grad():
         for m in model.modules():
             if isinstance(m, H.RMSNorm):
@@ -52,7 +52,7 @@ def test_hunyuan_swap_in_matches_eager_model(head_dim):
     counts = S.swap_in(wrapped, blocks=True)
     # LayerNorms: norm1.norm, norm1_context.norm, norm2, norm2_context, single norm.norm, norm_out.norm; modulate attributes of
     # the three AdaLayerNormZero[Single]; the gate method of each block; q/k (+ added q/k) RMSNorms; two processors
-    assert counts == {"rmsnorm": 6, "layernorm": 6, "modulate": 3, "gate": 2, "block": 1, "attention": 0,
+    assert counts == {"rmsnorm": 6, "layernorm": 6, "modulate": 3, "gate": 2, "block": 2, "attention": 0,
                       "processor": 2}, counts
     dbl, sgl = model.transformer_blocks[0], model.single_transformer_blocks[0]
     assert isinstance(dbl.norm2, S.DeferredLayerNorm) and isinstance(dbl.norm2_context, S.DeferredLayerNorm)
@@ -68,6 +68,35 @@ def test_hunyuan_swap_in_matches_eager_model(head_dim):
     assert worst[0] < 2e-2, worst
     again = S.swap_in(wrapped, blocks=True)
     assert not any(again.values()), again                      # idempotent
+
+
+def test_single_stream_blocks_stop_copying_the_token_sequence(monkeypatch):
+    """Two single-stream blocks in a row after swap_in(blocks=True): the latent and text tokens are
+    re-joined without a copy wherever the halves come from this module's own split (block to block,
+    block to processor, processor to block); only the very first join, of the two separate streams
+    leaving the double-stream block, concatenates.  Output and gradients as in eager."""
+    from teletron_amd import swap_in as S
+    model, inputs, rotary, dy = make_model_and_inputs(seed=7, head_dim=128, n_single=2)
+    wrapped = WithRotary(model, rotary)
+    out_e, gin_e, gp_e = run(wrapped, inputs, dy)
+    counts = S.swap_in(wrapped, blocks=True)
+    assert counts["block"] == 3 and counts["processor"] == 3, counts
+    original, seen = S.join_tokens, []
+
+    def counting(a, b):
+        r = original(a, b)
+        seen.append(r is getattr(a, "_tt_whole", None))
+        return r
+
+    monkeypatch.setattr(S, "join_tokens", counting)
+    out_f, gin_f, gp_f = run(wrapped, inputs, dy)
+    # per single-stream block: block entry, processor entry, after the attention
+    assert seen == [False, True, True, True, True, True], seen
+    assert rel(out_f, out_e) < 5e-3, rel(out_f, out_e)
+    for a, b in zip(gin_f, gin_e):
+        assert rel(a, b) < 2e-2
+    worst = max((rel(gp_f[n], gp_e[n]), n) for n in gp_e)
+    assert worst[0] < 2e-2, worst
 
 
 def test_fused_processor_against_original_processor():

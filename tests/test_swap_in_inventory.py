@@ -156,7 +156,7 @@ def patched_sites(root, before):
         elif "forward" in m.__dict__:
             kind = {"RMSNorm": "rmsnorm", "GateModule": "gate-module", "ContextParallelGateModule": "gate-module",
                     "DiTBlock": "block", "ContextParallelWanDitBlock": "block", "SelfAttention": "attention",
-                    "HunyuanVideoTransformerBlock": "block"}
+                    "HunyuanVideoTransformerBlock": "block", "HunyuanVideoSingleTransformerBlock": "block"}
             got[path] = kind.get(type(m).__name__, "unexpected forward on " + type(m).__name__)
         if hasattr(m.__dict__.get("gate"), "__wrapped__"):
             got[path + "#gate"] = "gate-method"
@@ -215,7 +215,7 @@ def test_swap_in_patches_every_recorded_site_and_nothing_else(blocks):
     counts = S.swap_in(root, [ns], blocks=blocks)
     got = patched_sites(root, before)
     if blocks:
-        want.update({"m0": "block", "m2": "block", "m0.self_attn": "attention", "m2.attn#processor": "processor",
+        want.update({"m0": "block", "m2": "block", "m3": "block", "m0.self_attn": "attention", "m2.attn#processor": "processor",
                      "m3.attn#processor": "processor"})
     assert got == want, sorted(set(got.items()) ^ set(want.items()))
     assert hasattr(ns.modulate, "__wrapped__")                 # DiTBlock calls the module-level modulate
@@ -277,11 +277,12 @@ def test_context_parallel_assignments_are_recognised(monkeypatch):
     counts = S.swap_in(root, blocks=True)
     assert counts["processor"] == 0                            # the context-parallel processors are not replaced
     assert counts["gate"] == 2 + 1 + 2 and counts["modulate"] == 3 + 1, counts      # methods + CP callable + GateModules
-    assert counts["block"] == 2          # the Wan block and the double-stream block, both on one rank
+    assert counts["block"] == 3          # the Wan block and both HunyuanVideo blocks on one rank
     root = assigned_model()
     monkeypatch.setattr(S, "_several_ranks", lambda: True)
     counts = S.swap_in(root, blocks=True)
-    assert counts["gate"] == 2 and counts["modulate"] == 1 and counts["block"] == 0, counts   # GateModules of the Wan block; norm1_context
+    # GateModules of the Wan block; norm1_context; the single-stream forward only drops copies (nothing to all-reduce)
+    assert counts["gate"] == 2 and counts["modulate"] == 1 and counts["block"] == 1, counts
     assert isinstance(root.m2.norm1, nn.LayerNorm) and isinstance(root.m0.norm1.norm, nn.LayerNorm)
     assert isinstance(root.m0.norm2, S.DeferredLayerNorm)      # inline modulation: row-local, no all-reduce involved
 
@@ -294,6 +295,7 @@ def test_replacement_forwards_keep_the_recorded_signatures():
              (S.fused_dit_block_forward, spec_of("ContextParallelWanDitBlock")["methods"]["forward"]),
              (S.fused_self_attention_forward, spec_of("SelfAttention")["methods"]["forward"]),
              (S.fused_hunyuan_block_forward, spec_of("HunyuanVideoTransformerBlock")["methods"]["forward"]),
+             (S.fused_hunyuan_single_block_forward, spec_of("HunyuanVideoSingleTransformerBlock")["methods"]["forward"]),
              (S.FusedHunyuanAttnProcessor.__call__, spec_of("HunyuanVideoAttnProcessor2_0")["methods"]["__call__"]),
              (S._fused_gate_forward, spec_of("GateModule")["methods"]["forward"]),
              (S._fused_rmsnorm_forward, spec_of("RMSNorm")["methods"]["forward"])]
@@ -319,3 +321,25 @@ def test_rotary_table_cache_follows_the_tensors_it_was_built_from():
     assert 2 not in cache.entries and 0 in cache.entries                  # ... and dropped with that object
     del cos, sin
     assert not cache.entries
+
+
+def test_join_tokens_returns_the_uncut_tensor_only_for_its_own_halves():
+    t = torch.randn(2, 7, 4, requires_grad=True) * 1.0
+    a, b = S.split_tokens(t, 3)
+    assert a.shape == (2, 4, 4) and b.shape == (2, 3, 4)
+    assert S.join_tokens(a, b) is t                                   # the halves, in place: no copy
+    assert torch.equal(S.join_tokens(b, a), torch.cat([b, a], dim=1)) and S.join_tokens(b, a) is not t   # wrong order
+    assert S.join_tokens(a.detach(), b) is not t                      # another tensor object carries no hint
+    assert S.join_tokens(a * 1.0, b) is not t
+    u = torch.randn(2, 7, 4)
+    c, d = S.split_tokens(u, 3)
+    assert S.join_tokens(a, d) is not t and torch.equal(S.join_tokens(a, d), torch.cat([a, d], dim=1))   # halves of two tensors
+    # gradients through the uncut tensor equal those through slicing and concatenating
+    w = torch.randn(2, 7, 4)
+    (g1,) = torch.autograd.grad((S.join_tokens(*S.split_tokens(t, 3)) * w).sum(), t, retain_graph=True)
+    (g2,) = torch.autograd.grad((torch.cat([t[:, :-3], t[:, -3:]], dim=1) * w).sum(), t)
+    assert torch.equal(g1, g2)
+    x = torch.randn(2, 7, 4)
+    p, q_ = S.split_tokens(x, 3)
+    p.mul_(2.0)                                                        # in place on a half: the whole tensor sees it
+    assert S.join_tokens(p, q_) is x and torch.equal(x[:, :4], p)
