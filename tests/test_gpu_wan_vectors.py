@@ -106,3 +106,35 @@ def test_fused_ops_against_the_reference_codes_numbers(name):
         else:       # the autograd Function hands the parameter gradient back in the parameter's dtype: bf16
             tol = 1e-3 * np.abs(f32[k]) + 1e-4 * np.sqrt(rows) + 2.0 ** -8 * np.abs(f32[k])
             assert np.all(np.abs(g - f32[k]) <= tol), (name, k, np.abs(g - f32[k]).max())
+
+
+def test_swapped_blocks_under_activation_checkpointing():
+    """WanModel.forward can run every block under torch.utils.checkpoint (use_reentrant=False,
+    wan_model.py:376-390): the swapped-in forwards are recomputed in backward and must give the very
+    same output and gradients as without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+    from teletron_amd import swap_in as S
+    inputs = W.case_inputs()
+    model = W.standin_case_model()
+    S.swap_in(model, namespaces=[W], blocks=True)
+
+    class Checkpointed(torch.nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, x, context, t_mod, t, freqs):
+            for block in self.inner.blocks:
+                x = checkpoint(block, x, context, t_mod, freqs, use_reentrant=False)
+            return self.inner.head(x, t)
+
+    try:
+        plain = W.run_case(model, inputs, DEV, torch.bfloat16)
+        ckpt = W.run_case(Checkpointed(model), inputs, DEV, torch.bfloat16)
+    finally:
+        W.modulate = W.modulate.__wrapped__ if hasattr(W.modulate, "__wrapped__") else W.modulate
+    assert torch.equal(plain[0], ckpt[0])
+    for a, b in zip(plain[1], ckpt[1]):
+        assert torch.equal(a, b)
+    for n, g in plain[2].items():
+        assert torch.equal(g, ckpt[2]["inner." + n]), n
