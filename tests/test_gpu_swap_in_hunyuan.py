@@ -99,6 +99,38 @@ def test_single_stream_blocks_stop_copying_the_token_sequence(monkeypatch):
     assert worst[0] < 2e-2, worst
 
 
+@pytest.mark.parametrize("reentrant", [False, True])
+def test_swapped_hunyuan_blocks_under_activation_checkpointing(reentrant):
+    """Every block under torch.utils.checkpoint, as the model's gradient checkpointing runs them
+    (hunyuan/model.py:919-951): recomputed forwards, and (reentrant) block outputs that are new tensor
+    objects, so the no-copy re-join falls back to concatenating; results as without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+    from teletron_amd import swap_in as S
+    model, inputs, rotary, dy = make_model_and_inputs(seed=9, head_dim=128, n_single=2)
+    S.swap_in(model, blocks=True)
+
+    class Checkpointed(nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, h, e, temb):
+            for blk in list(self.inner.transformer_blocks) + list(self.inner.single_transformer_blocks):
+                h, e = checkpoint(blk, h, e, temb, None, rotary, use_reentrant=reentrant)
+            return torch.cat([self.inner.norm_out(h, temb), e], dim=1)
+
+    plain = run(WithRotary(model, rotary), inputs, dy)
+    ckpt = run(Checkpointed(model), inputs, dy)
+    # recomputation is deterministic; reentrant checkpointing sums the gradients of an input shared by
+    # several blocks (temb) in another order, hence bf16-rounding differences there
+    same = (lambda a, b: torch.equal(a, b)) if not reentrant else (lambda a, b: rel(a, b) < 5e-3)
+    assert same(plain[0], ckpt[0])
+    for a, b in zip(plain[1], ckpt[1]):
+        assert same(a, b)
+    for n, g in plain[2].items():
+        assert same(g, ckpt[2][n.replace("model.", "inner.", 1)]), n
+
+
 def test_fused_processor_against_original_processor():
     """The processor on its own, latent / text split included: the single-stream attention with the
     text tokens appended (no rotation for them) and the double-stream one."""
