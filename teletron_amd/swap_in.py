@@ -271,9 +271,17 @@ class _RotaryTableCache:
     def __init__(self):
         self.entries = {}
 
+    @staticmethod
+    def _versions(cos, sin):
+        try:
+            return cos._version, sin._version
+        except RuntimeError:        # tensors made under torch.inference_mode() keep no version counter:
+            return None             # the same objects are then taken to hold the same values
+
     def get(self, cos: torch.Tensor, sin: torch.Tensor, extra_tokens: int) -> torch.Tensor:
         e = self.entries.get(extra_tokens)
-        if e is not None and e[0]() is cos and e[1]() is sin and e[2] == (cos._version, sin._version):
+        versions = self._versions(cos, sin)
+        if e is not None and e[0]() is cos and e[1]() is sin and e[2] == versions:
             return e[3]
         table = rope_table_from_cos_sin(cos, sin, extra_tokens=extra_tokens)
 
@@ -282,7 +290,7 @@ class _RotaryTableCache:
             if held is not None and ref in (held[0], held[1]):
                 del self.entries[key]
 
-        self.entries[extra_tokens] = (weakref.ref(cos, drop), weakref.ref(sin, drop), (cos._version, sin._version), table)
+        self.entries[extra_tokens] = (weakref.ref(cos, drop), weakref.ref(sin, drop), versions, table)
         return table
 
 

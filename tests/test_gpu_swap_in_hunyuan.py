@@ -131,6 +131,23 @@ def test_swapped_hunyuan_blocks_under_activation_checkpointing(reentrant):
         assert same(g, ckpt[2][n.replace("model.", "inner.", 1)]), n
 
 
+def test_swapped_model_under_inference_mode():
+    """Generation runs under torch.inference_mode(): tensors made there keep no version counter and
+    no autograd state; the swapped model must run and give the no_grad result."""
+    from teletron_amd import swap_in as S
+    model, inputs, _, _ = make_model_and_inputs(seed=11, head_dim=128, n_single=2)
+    S.swap_in(model, blocks=True)
+    with torch.inference_mode():
+        g = torch.Generator().manual_seed(12)
+        ang = 3.0 * torch.randn(inputs[0].shape[1], 64, generator=g)
+        rotary = (ang.cos().repeat_interleave(2, dim=1).to(DEV), ang.sin().repeat_interleave(2, dim=1).to(DEV))
+        out_i = model(*inputs, *rotary)
+        out_i2 = model(*inputs, *rotary)            # second pass: the cached rotary table
+    with torch.no_grad():
+        out_n = model(*inputs, rotary[0].clone(), rotary[1].clone())
+    assert torch.equal(out_i, out_n) and torch.equal(out_i2, out_n)
+
+
 def test_fused_processor_against_original_processor():
     """The processor on its own, latent / text split included: the single-stream attention with the
     text tokens appended (no rotation for them) and the double-stream one."""

@@ -138,3 +138,22 @@ def test_swapped_blocks_under_activation_checkpointing():
         assert torch.equal(a, b)
     for n, g in plain[2].items():
         assert torch.equal(g, ckpt[2]["inner." + n]), n
+
+
+def test_swapped_wan_blocks_under_inference_mode():
+    """Generation runs under torch.inference_mode(); the swapped-in forwards must work on tensors
+    that carry no autograd state and give the no_grad result."""
+    from teletron_amd import swap_in as S
+    x, context, t_mod, t, angles, _ = W.case_inputs()
+    model = W.standin_case_model().to(DEV).to(torch.bfloat16)
+    S.swap_in(model, namespaces=[W], blocks=True)
+    try:
+        args = [v.to(DEV).to(torch.bfloat16) for v in (x, context, t_mod, t)]
+        with torch.inference_mode():
+            out_i = model(*[a.clone() for a in args], W.freqs_from_angles(angles.to(DEV)))
+        with torch.no_grad():
+            out_n = model(*args, W.freqs_from_angles(angles.to(DEV)))
+    finally:
+        W.modulate = W.modulate.__wrapped__ if hasattr(W.modulate, "__wrapped__") else W.modulate
+    assert torch.equal(out_i, out_n)
+    assert rel(out_n.float().cpu().numpy(), GOLD["out"]) < 2e-2
