@@ -247,15 +247,27 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
     return GateResidualFunction.apply(x, gate_mlp, self.ffn(input_x))
 
 
+def _projection_dtype(x: torch.Tensor) -> torch.dtype:
+    """dtype that ``nn.Linear(x)`` returns: the autocast dtype while autocast is on, else x's own."""
+    if torch.is_autocast_enabled(x.device.type):
+        return torch.get_autocast_dtype(x.device.type)
+    return x.dtype
+
+
 def fused_self_attention_forward(self, x, freqs):
     """``SelfAttention.forward`` (``wan_model.py:153-160``) with ``norm_q`` / ``norm_k`` and the
     ``rope_apply`` that follows each of them in one kernel per tensor; projections and the attention
     module (possibly wrapped for context parallelism) are used as they are."""
-    q, k = self.q(x), self.k(x)
-    head_dim = q.shape[-1] // self.num_heads
-    if not (q.is_cuda and q.dtype == torch.bfloat16 and q.shape[-1] > 256 and head_dim % 8 == 0 and head_dim <= 256
-            and q.dim() >= 2 and freqs.shape[0] == q.shape[-2] and _same_dtype(q, self.norm_q.weight, self.norm_k.weight)):
+    width = getattr(self.q, "out_features", x.shape[-1])
+    head_dim = width // self.num_heads
+    # decided before the projections run, so that the original forward does not repeat them
+    if not (x.is_cuda and _projection_dtype(x) == torch.bfloat16 and width > 256 and width % self.num_heads == 0
+            and head_dim % 8 == 0 and head_dim <= 256 and x.dim() >= 2 and freqs.shape[0] == x.shape[-2]
+            and self.norm_q.weight.dtype == torch.bfloat16 and self.norm_k.weight.dtype == torch.bfloat16):
         return type(self).forward(self, x, freqs)
+    q, k = self.q(x), self.k(x)
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or q.shape[-1] != width or k.shape[-1] != width:
+        return type(self).forward(self, x, freqs)          # a projection that is not a plain nn.Linear
     table = ops._check_freqs(freqs.detach(), q, head_dim)          # converted once, shared by q and k
     q = RMSNormRopeFunction.apply(q, self.norm_q.weight, table, self.norm_q.eps, self.num_heads)
     k = RMSNormRopeFunction.apply(k, self.norm_k.weight, table, self.norm_k.eps, self.num_heads)

@@ -157,3 +157,34 @@ def test_swapped_wan_blocks_under_inference_mode():
         W.modulate = W.modulate.__wrapped__ if hasattr(W.modulate, "__wrapped__") else W.modulate
     assert torch.equal(out_i, out_n)
     assert rel(out_n.float().cpu().numpy(), GOLD["out"]) < 2e-2
+
+
+def test_fp32_master_weights_under_autocast_stay_on_the_original_code():
+    """Parameters kept in float32 and the model run under torch.autocast(bfloat16): the eager code
+    promotes (RMSNorm output * fp32 weight is fp32, LayerNorm runs in fp32), which the bf16 kernels do
+    not reproduce, so every swapped site must hand such inputs to the original code: bit-identical
+    output and gradients before and after swap_in, and no projection computed twice."""
+    from teletron_amd import swap_in as S
+    inputs = W.case_inputs()
+    model = W.standin_case_model()
+
+    def run_autocast():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            return W.run_case(model, inputs, DEV, torch.float32)
+
+    eager = run_autocast()
+    counts = S.swap_in(model, namespaces=[W], blocks=True)
+    assert counts["block"] == 2 and counts["attention"] == 2
+    calls = []
+    hook = model.blocks[0].self_attn.q.register_forward_hook(lambda *a: calls.append(1))
+    try:
+        swapped = run_autocast()
+    finally:
+        hook.remove()
+        W.modulate = W.modulate.__wrapped__ if hasattr(W.modulate, "__wrapped__") else W.modulate
+    assert len(calls) == 1, calls
+    assert torch.equal(eager[0], swapped[0])
+    for a, b in zip(eager[1], swapped[1]):
+        assert torch.equal(a, b)
+    for n in eager[2]:
+        assert torch.equal(eager[2][n], swapped[2][n]), n
