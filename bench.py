@@ -451,8 +451,8 @@ def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3
             "relative_output_difference": diff, "swapped": counts}
 
 
-def hunyuan_block_demo(n_img=16384, n_txt=256, n_single=3, heads=24, head_dim=128, iters=4):
-    """Whole-block view for HunyuanVideo (--block-demo): `n_single` single-stream blocks in a row, built
+def hunyuan_block_demo(kind="single", n_img=16384, n_txt=256, n_blocks=3, heads=24, head_dim=128, iters=4):
+    """Whole-block view for HunyuanVideo (--block-demo): `n_blocks` single- or double-stream blocks in a row, built
     from the stand-ins the swap-in tests use (tests/hunyuan_standins.py: the call pattern of
     teletron/models/hunyuan/model.py:64-170,472-583 around nn.Linear and torch SDPA), forward +
     backward in eager PyTorch, after swap_in() and after swap_in(blocks=True) (fused per-head norm +
@@ -465,8 +465,8 @@ def hunyuan_block_demo(n_img=16384, n_txt=256, n_single=3, heads=24, head_dim=12
 
     def build():
         torch.manual_seed(0)
-        return torch.nn.ModuleList([H.HunyuanVideoSingleTransformerBlock(heads, head_dim, mlp_ratio=4)
-                                    for _ in range(n_single)]).to(dev).to(bf)
+        cls = H.HunyuanVideoSingleTransformerBlock if kind == "single" else H.HunyuanVideoTransformerBlock
+        return torch.nn.ModuleList([cls(heads, head_dim, mlp_ratio=4) for _ in range(n_blocks)]).to(dev).to(bf)
 
     g = torch.Generator(device=dev).manual_seed(1)
     rnd = lambda *shape: torch.randn(*shape, device=dev, generator=g)
@@ -500,7 +500,8 @@ def hunyuan_block_demo(n_img=16384, n_txt=256, n_single=3, heads=24, head_dim=12
     counts = S.swap_in(m, blocks=True)
     blocks_ms, out_f = timed(m)
     diff = float((out_f.double() - out_e.double()).norm() / out_e.double().norm())
-    return {"block": f"{n_single} HunyuanVideoSingleTransformerBlock stand-ins, dim {dim}, {heads} heads, "
+    name = "HunyuanVideoSingleTransformerBlock" if kind == "single" else "HunyuanVideoTransformerBlock"
+    return {"block": f"{n_blocks} {name} stand-ins, dim {dim}, {heads} heads, "
                      f"{n_img} latent + {n_txt} text tokens, bf16",
             "eager_ms": round(eager_ms, 2), "swap_in_ms": round(swapped_ms, 2), "swap_in_blocks_ms": round(blocks_ms, 2),
             "speedup": round(eager_ms / blocks_ms, 3), "relative_output_difference": diff, "swapped": counts}
@@ -681,7 +682,8 @@ def main():
     if also:
         out["also"] = also
     if args.block_demo:
-        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824), hunyuan_block_demo()]
+        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824), hunyuan_block_demo("single"),
+                             hunyuan_block_demo("double", n_blocks=2)]
     if args.calibrate_copy:
         src = torch.empty(w.elements, dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
         dst = torch.empty_like(src)
