@@ -237,8 +237,11 @@ class GpuWorkload:
             t = statistics.median(e[0].elapsed_time(e[1]) for e in ev[3:]) * 1e-3
             return {"read": 1, "write": 1, "copy": 2, "2r1w": 3}[mix] * nbytes / t / 1e9
 
+        # the bare copy depends on where the two buffers lie relative to one another (period 128 MiB:
+        # fast over one half of it, up to 25 % slower over the other); say where these lie
+        placement = [round(((s["x"].data_ptr() - s["y"].data_ptr()) % (128 << 20)) / 2 ** 20, 1) for s in self.sets]
         return {"copy": timed("copy"), "two_reads_one_write": timed("2r1w"),
-                "read_only": timed("read"), "write_only": timed("write")}
+                "read_only": timed("read"), "write_only": timed("write"), "copy_in_minus_out_mod_128MiB": placement}
 
     def run(self, steps, warmup):
         """Returns wall seconds per step and per-kernel mean microseconds from HIP events."""
@@ -658,7 +661,10 @@ def main():
         "read_only": round(c["read_only"], 1), "write_only": round(c["write_only"], 1),
         "forward_frac_of_copy": round(r["fwd_gbps"] / c["copy"], 4),
         "backward_frac_of_two_reads_one_write": round(r["bwd_gbps"] / c["two_reads_one_write"], 4),
-        "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers"}
+        "copy_in_minus_out_mod_128MiB": c["copy_in_minus_out_mod_128MiB"],
+        "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers; the bare "
+                "copy is up to 25 % slower when (x - y) mod 128 MiB falls in about [104, 128) or [0, 38) MiB, the "
+                "normalisation kernels are not"}
     if not args.no_eager_gpu:
         ms = eager_gpu(w)
         if ms:
