@@ -3,12 +3,12 @@
 The compute path is hand-written HIP for gfx950 in ``libteletron_op.so`` (C ABI,
 ``include/teletron_op.h``); Python only validates, allocates and launches.
 """
-from .functional import (AdaLNModelFunction, FusedAdaLN, FusedGate, FusedRMSNorm, GateResidualFunction,
+from .functional import (AdaLNGradReduceFunction, AdaLNModelFunction, FusedAdaLN, GateResidualGradReduceFunction, FusedGate, FusedRMSNorm, GateResidualFunction,
                          RMSNormModelFunction, RMSNormRopeFunction, RMSNormRopeHeadsFunction, ResidualNormFunction, adaln_modulate,
                          residual_adaln, residual_layer_norm, rms_norm, rope_table_from_cos_sin)
 from . import cabi, ops, swap_in, workloads
 
-__all__ = ["AdaLNModelFunction", "RMSNormModelFunction", "GateResidualFunction", "RMSNormRopeFunction", "FusedAdaLN", "FusedRMSNorm", "FusedGate",
+__all__ = ["AdaLNModelFunction", "AdaLNGradReduceFunction", "GateResidualGradReduceFunction", "RMSNormModelFunction", "GateResidualFunction", "RMSNormRopeFunction", "FusedAdaLN", "FusedRMSNorm", "FusedGate",
            "ResidualNormFunction", "RMSNormRopeHeadsFunction", "rope_table_from_cos_sin", "residual_adaln", "residual_layer_norm", "adaln_modulate", "rms_norm", "cabi", "ops", "swap_in", "workloads", "install_reference_modules"]
 
 

@@ -27,31 +27,60 @@ from torch.autograd import Function
 from . import ops
 
 
+def _adaln_forward(ctx, x, scale, shift, epsilon, cols):
+    if x.numel() % cols != 0 or x.shape[-1] != cols:
+        raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols}")
+    ctx.eps = float(epsilon)
+    ctx.scale_meta = (scale.shape, scale.dtype)
+    ctx.shift_meta = (shift.shape, shift.dtype)
+    x = x.contiguous()
+    scale_c = scale.detach().to(torch.bfloat16).contiguous()
+    y = ops.adaln_forward(x, scale_c, shift.detach(), ctx.eps)
+    ctx.save_for_backward(x, scale_c)
+    return y
+
+
+def _adaln_backward(ctx, grad_output, grad_reduce=None):
+    x, scale_c = ctx.saved_tensors
+    dx, grads = ops.adaln_backward_packed(grad_output.contiguous(), x, scale_c, ctx.eps)
+    if grad_reduce is not None:
+        grad_reduce(grads)                  # fp32 [2, n_batches, C]: dscale and dshift in ONE exchange, before the cast
+    (sc_shape, sc_dtype), (sh_shape, sh_dtype) = ctx.scale_meta, ctx.shift_meta
+    if sc_dtype == sh_dtype:
+        grads = grads.to(sc_dtype)          # both parameter gradients in one cast
+    dx = dx if ctx.needs_input_grad[0] else None
+    dscale = grads[0].to(sc_dtype).reshape(sc_shape) if ctx.needs_input_grad[1] else None
+    dshift = grads[1].to(sh_dtype).reshape(sh_shape) if ctx.needs_input_grad[2] else None
+    return dx, dscale, dshift
+
+
 class AdaLNModelFunction(Function):
     @staticmethod
     def forward(ctx, x, scale, shift, epsilon, cols):
-        if x.numel() % cols != 0 or x.shape[-1] != cols:
-            raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols}")
-        ctx.eps = float(epsilon)
-        ctx.scale_meta = (scale.shape, scale.dtype)
-        ctx.shift_meta = (shift.shape, shift.dtype)
-        x = x.contiguous()
-        scale_c = scale.detach().to(torch.bfloat16).contiguous()
-        y = ops.adaln_forward(x, scale_c, shift.detach(), ctx.eps)
-        ctx.save_for_backward(x, scale_c)
-        return y
+        return _adaln_forward(ctx, x, scale, shift, epsilon, cols)
 
     @staticmethod
     def backward(ctx, grad_output):
-        x, scale_c = ctx.saved_tensors
-        dx, grads = ops.adaln_backward_packed(grad_output.contiguous(), x, scale_c, ctx.eps)
-        (sc_shape, sc_dtype), (sh_shape, sh_dtype) = ctx.scale_meta, ctx.shift_meta
-        if sc_dtype == sh_dtype:
-            grads = grads.to(sc_dtype)          # both parameter gradients in one cast
-        dx = dx if ctx.needs_input_grad[0] else None
-        dscale = grads[0].to(sc_dtype).reshape(sc_shape) if ctx.needs_input_grad[1] else None
-        dshift = grads[1].to(sh_dtype).reshape(sh_shape) if ctx.needs_input_grad[2] else None
-        return dx, dscale, dshift, None, None
+        return (*_adaln_backward(ctx, grad_output), None, None)
+
+
+class AdaLNGradReduceFunction(Function):
+    """``AdaLNModelFunction`` for a sequence-sharded (context-parallel) model: every rank holds a slice
+    of the rows, so the gradients of ``scale`` / ``shift`` must be summed over the ranks, which is what
+    ``ModulateWithCPGradReduce`` does with two all-reduces of bf16 ``[B, 1, C]`` tensors
+    (``teletron/core/context_parallel/layers.py:39-53``).  ``grad_reduce`` is any callable that sums an
+    fp32 tensor over the group in place (``lambda t: torch.distributed.all_reduce(t, group=cp_group)``);
+    it is called once per backward, on the fp32 ``[2, B, C]`` tensor holding both gradients, before
+    the cast to the parameters' dtype.  ``apply(x, scale, shift, epsilon, cols, grad_reduce)``."""
+
+    @staticmethod
+    def forward(ctx, x, scale, shift, epsilon, cols, grad_reduce):
+        ctx.grad_reduce = grad_reduce
+        return _adaln_forward(ctx, x, scale, shift, epsilon, cols)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return (*_adaln_backward(ctx, grad_output, ctx.grad_reduce), None, None, None)
 
 
 class RMSNormModelFunction(Function):
@@ -145,6 +174,27 @@ def rope_table_from_cos_sin(cos: torch.Tensor, sin: torch.Tensor, extra_tokens: 
     return table.contiguous()
 
 
+def _gate_forward(ctx, x, gate, residual):
+    ctx.gate_meta = (gate.shape, gate.dtype)
+    gate_c = gate.detach().to(torch.bfloat16).contiguous()
+    residual = residual.contiguous()
+    ctx.save_for_backward(gate_c, residual)
+    return ops.gate_residual_forward(x.contiguous(), gate_c, residual)
+
+
+def _gate_backward(ctx, grad_output, grad_reduce=None):
+    gate_c, residual = ctx.saved_tensors
+    g_shape, g_dtype = ctx.gate_meta
+    if not (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]):
+        return grad_output, None, None
+    dres, dgate = ops.gate_residual_backward(grad_output.contiguous(), gate_c, residual)
+    if grad_reduce is not None and ctx.needs_input_grad[1]:
+        grad_reduce(dgate)                  # fp32 [n_batches, C], before the cast
+    return (grad_output if ctx.needs_input_grad[0] else None,
+            dgate.to(g_dtype).reshape(g_shape) if ctx.needs_input_grad[1] else None,
+            dres if ctx.needs_input_grad[2] else None)
+
+
 class GateResidualFunction(Function):
     """``x + gate * residual`` with the hand-written backward of ``GateWithGradReduce``
     (``teletron/core/context_parallel/layers.py:24-36``) on one GPU: returns
@@ -152,22 +202,26 @@ class GateResidualFunction(Function):
 
     @staticmethod
     def forward(ctx, x, gate, residual):
-        ctx.gate_meta = (gate.shape, gate.dtype)
-        gate_c = gate.detach().to(torch.bfloat16).contiguous()
-        residual = residual.contiguous()
-        ctx.save_for_backward(gate_c, residual)
-        return ops.gate_residual_forward(x.contiguous(), gate_c, residual)
+        return _gate_forward(ctx, x, gate, residual)
 
     @staticmethod
     def backward(ctx, grad_output):
-        gate_c, residual = ctx.saved_tensors
-        g_shape, g_dtype = ctx.gate_meta
-        if not (ctx.needs_input_grad[1] or ctx.needs_input_grad[2]):
-            return grad_output, None, None
-        dres, dgate = ops.gate_residual_backward(grad_output.contiguous(), gate_c, residual)
-        return (grad_output if ctx.needs_input_grad[0] else None,
-                dgate.to(g_dtype).reshape(g_shape) if ctx.needs_input_grad[1] else None,
-                dres if ctx.needs_input_grad[2] else None)
+        return _gate_backward(ctx, grad_output)
+
+
+class GateResidualGradReduceFunction(Function):
+    """``GateResidualFunction`` whose gate gradient is summed over the ranks of a sequence-sharded
+    model, as ``GateWithGradReduce`` does (``context_parallel/layers.py:31-36``): ``grad_reduce`` is
+    called on the fp32 ``[B, C]`` gradient before the cast.  ``apply(x, gate, residual, grad_reduce)``."""
+
+    @staticmethod
+    def forward(ctx, x, gate, residual, grad_reduce):
+        ctx.grad_reduce = grad_reduce
+        return _gate_forward(ctx, x, gate, residual)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return (*_gate_backward(ctx, grad_output, ctx.grad_reduce), None)
 
 
 class ResidualNormFunction(Function):

@@ -44,11 +44,13 @@ ships no code that performs the swap.  This module does it by patching *instance
   :class:`FusedHunyuanAttnProcessor`, which runs ``norm_q`` / ``norm_k`` and the rotary embedding
   after them as one kernel per tensor (text tokens appended to the latent ones take no rotation).
 
-Single-GPU semantics only: ``modulate_with_cp_grad_reduce`` / ``gate_with_cp_grad_reduce``
-all-reduce their parameter gradients over the context-parallel group
+Context parallelism: ``modulate_with_cp_grad_reduce`` / ``gate_with_cp_grad_reduce`` all-reduce
+their parameter gradients over the context-parallel group
 (``core/context_parallel/layers.py:31-36,46-53``); with a group of size 1 that is the identity,
-which is what the fused ops return.  While ``torch.distributed`` runs with more than one rank
-these callables (and the context-parallel block's forward) are therefore left as they are.
+which is what the plain fused ops return.  While ``torch.distributed`` runs with more than one rank
+these callables are left as they are unless ``swap_in`` is told how to reduce (``cp_grad_reduce``),
+in which case they are replaced by fused ops that pass their fp32 parameter gradients through that
+callable; the whole-block forwards are not installed on context-parallel blocks then.
 """
 from __future__ import annotations
 
@@ -62,7 +64,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .functional import (AdaLNModelFunction, GateResidualFunction, RMSNormModelFunction, RMSNormRopeFunction,
+from .functional import (AdaLNGradReduceFunction, AdaLNModelFunction, GateResidualFunction,
+                         GateResidualGradReduceFunction, RMSNormModelFunction, RMSNormRopeFunction,
                          RMSNormRopeHeadsFunction, adaln_modulate, residual_adaln, residual_layer_norm,
                          rope_table_from_cos_sin)
 
@@ -123,30 +126,40 @@ class DeferredNorm:
             "`modulate(...)` or used as `norm(x) * (1 + scale) + shift`; call .materialize() for anything else")
 
 
-def modulate_token(token: DeferredNorm, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+def modulate_token(token: DeferredNorm, shift: torch.Tensor, scale: torch.Tensor,
+                   grad_reduce: Optional[Callable] = None) -> torch.Tensor:
     x = token.x
     if not _same_dtype(x, shift, scale):      # wider modulation: the eager expression, which promotes
+        if grad_reduce is not None:
+            raise TypeError("the gradient-reducing fused modulation needs shift / scale in the activation's dtype")
         return token.materialize() * (1 + scale) + shift
+    if grad_reduce is not None:
+        return AdaLNGradReduceFunction.apply(x, scale, shift, token.eps, x.shape[-1], grad_reduce)
     return AdaLNModelFunction.apply(x, scale, shift, token.eps, x.shape[-1])
 
 
-def fused_modulate(original: Callable) -> Callable:
-    """Wrap a ``modulate(x, shift, scale)`` callable: tokens take the fused kernel, tensors the original."""
+def fused_modulate(original: Callable, grad_reduce: Optional[Callable] = None) -> Callable:
+    """Wrap a ``modulate(x, shift, scale)`` callable: tokens take the fused kernel, tensors the original.
+    ``grad_reduce`` (for a callable that sums its parameter gradients over a process group, see
+    :func:`swap_in`) is applied to the fused op's fp32 parameter gradients."""
 
     def modulate(x, shift, scale):
         if isinstance(x, DeferredNorm):
-            return modulate_token(x, shift, scale)
+            return modulate_token(x, shift, scale, grad_reduce)
         return original(x, shift, scale)
 
     modulate.__wrapped__ = original
     return modulate
 
 
-def fused_gate(original: Callable) -> Callable:
-    """Wrap a ``gate(x, gate, residual)`` callable: bf16 GPU tensors take the fused kernel."""
+def fused_gate(original: Callable, grad_reduce: Optional[Callable] = None) -> Callable:
+    """Wrap a ``gate(x, gate, residual)`` callable: bf16 GPU tensors take the fused kernel
+    (``grad_reduce`` as in :func:`fused_modulate`)."""
 
     def gate(x, gate, residual):
         if _gate_fusable(x, gate, residual):
+            if grad_reduce is not None:
+                return GateResidualGradReduceFunction.apply(x, gate, residual, grad_reduce)
             return GateResidualFunction.apply(x, gate, residual)
         return original(x, gate, residual)
 
@@ -209,6 +222,9 @@ def _gate_fusable(x, gate, residual) -> bool:
 
 def _fused_gate_forward(self, x, gate, residual):
     if _gate_fusable(x, gate, residual):
+        grad_reduce = self.__dict__.get("_tt_grad_reduce")
+        if grad_reduce is not None:
+            return GateResidualGradReduceFunction.apply(x, gate, residual, grad_reduce)
         return GateResidualFunction.apply(x, gate, residual)
     return type(self).forward(self, x, gate, residual)
 
@@ -477,11 +493,17 @@ def _is_dit_block(m: nn.Module) -> bool:
 
 
 def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool = True, adaln: bool = True,
-            gate: bool = True, blocks: bool = False) -> dict:
+            gate: bool = True, blocks: bool = False, cp_grad_reduce: Optional[Callable] = None) -> dict:
     """Patch ``model`` in place.  ``namespaces`` are Python modules (e.g. the imported
     ``teletron.models.wan.wan_model``) whose module-level ``modulate`` function should learn about
     tokens.  ``blocks`` also replaces the forward of whole DiT blocks (see the module docstring).
-    Returns counts of what was swapped."""
+    ``cp_grad_reduce``: for a sequence-sharded (context-parallel) model, a callable that sums an fp32
+    tensor over the context-parallel group in place, e.g.
+    ``lambda t: torch.distributed.all_reduce(t, group=mpu.get_context_parallel_group())``.  With it the
+    ``*_with_cp_grad_reduce`` callables and ``ContextParallelGateModule`` are replaced as well, by fused
+    ops that hand their fp32 parameter gradients to it (one exchange per op instead of the reference's
+    one per gradient, ``core/context_parallel/layers.py:31-36,46-53``); without it they are left alone
+    while more than one rank runs.  Returns counts of what was swapped."""
     counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0, "attention": 0, "processor": 0}
     for ns in namespaces:
         fn = getattr(ns, "modulate", None)
@@ -492,10 +514,13 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
         if rmsnorm and _is_rmsnorm(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(_fused_rmsnorm_forward, module)
             counts["rmsnorm"] += 1
-        if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__ \
-                and not (type(module).__name__ == "ContextParallelGateModule" and _several_ranks()):
-            module.forward = types.MethodType(_fused_gate_forward, module)
-            counts["gate"] += 1
+        if gate and type(module).__name__ in GATE_CLASSES and "forward" not in module.__dict__:
+            cp = type(module).__name__ == "ContextParallelGateModule"
+            if not (cp and cp_grad_reduce is None and _several_ranks()):
+                if cp and cp_grad_reduce is not None:
+                    module.__dict__["_tt_grad_reduce"] = cp_grad_reduce
+                module.forward = types.MethodType(_fused_gate_forward, module)
+                counts["gate"] += 1
         if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
             module.forward = types.MethodType(fused_dit_block_forward, module)
             counts["block"] += 1
@@ -510,9 +535,11 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
             counts["attention"] += 1
         if gate and type(module).__name__ in GATE_METHOD_OWNERS:
             fn = getattr(module, "gate", None)
+            cp = _is_cp_callable("gate", fn)
             if (callable(fn) and not isinstance(fn, nn.Module) and not hasattr(fn, "__wrapped__")
-                    and not (_is_cp_callable("gate", fn) and _several_ranks())):
-                module.gate = fused_gate(fn)        # instance attribute: shadows the method, as parallel_model.py:241 does
+                    and not (cp and cp_grad_reduce is None and _several_ranks())):
+                # instance attribute: shadows the method, as parallel_model.py:241 does
+                module.gate = fused_gate(fn, cp_grad_reduce if cp else None)
                 counts["gate"] += 1
         if blocks and rmsnorm and type(getattr(module, "processor", None)).__name__ == HUNYUAN_PROCESSOR \
                 and all(hasattr(module, a) for a in ("to_q", "to_k", "to_v", "heads", "norm_q", "norm_k", "add_q_proj")):
@@ -520,20 +547,22 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
             counts["processor"] += 1
         if adaln and type(module).__name__ in ADALN_OWNER_CLASSES:
             # The *_with_cp_grad_reduce callables all-reduce their parameter gradients over the
-            # context-parallel group; they are only replaced where that is the identity.  An owner
-            # whose modulation goes through one of them then keeps its LayerNorms as well.
+            # context-parallel group; they are only replaced where that is the identity or where the
+            # caller has said how to reduce.  An owner whose modulation goes through one of them and
+            # cannot be replaced keeps its LayerNorms as well.
             attrs = [(a, getattr(module, a, None)) for a in MODULATE_ATTRS + (GATE_ATTRS if gate else ())]
             attrs = [(a, fn) for a, fn in attrs if callable(fn) and not isinstance(fn, nn.Module)]
-            if _several_ranks() and any(_is_cp_callable(a, fn) for a, fn in attrs):
+            if cp_grad_reduce is None and _several_ranks() and any(_is_cp_callable(a, fn) for a, fn in attrs):
                 continue
             for attr, fn in attrs:
                 if hasattr(fn, "__wrapped__"):
                     continue
+                hook = cp_grad_reduce if _is_cp_callable(attr, fn) else None
                 if attr in GATE_ATTRS:
-                    setattr(module, attr, fused_gate(fn))
+                    setattr(module, attr, fused_gate(fn, hook))
                     counts["gate"] += 1
                 else:
-                    setattr(module, attr, fused_modulate(fn))
+                    setattr(module, attr, fused_modulate(fn, hook))
                     counts["modulate"] += 1
             for attr in ADALN_NORM_ATTRS:
                 ln = getattr(module, attr, None)

@@ -312,3 +312,106 @@ def test_deferred_norm_refuses_other_uses():
     ref = torch.nn.functional.layer_norm(x, (64,), eps=1e-6)
     assert torch.equal(tok.materialize(), ref)
     assert torch.equal(ln(x.float()), torch.nn.functional.layer_norm(x.float(), (64,), eps=1e-6))  # non-bf16: eager
+
+
+def test_gradient_reducing_variants_hand_fp32_parameter_gradients_to_the_hook():
+    """AdaLNGradReduceFunction / GateResidualGradReduceFunction: the hook sees the fp32 parameter
+    gradients (both AdaLN gradients in one tensor) before the cast.  A hook that doubles them stands
+    for two ranks holding the same rows: the result must be exactly twice the single-rank gradient."""
+    from teletron_amd import (AdaLNGradReduceFunction, AdaLNModelFunction, GateResidualFunction,
+                              GateResidualGradReduceFunction)
+    g = torch.Generator().manual_seed(21)
+    mk = lambda *s, scale=1.0: (scale * torch.randn(*s, generator=g)).to(torch.bfloat16).to(DEV)
+    x, dy, r = mk(2, 50, 512), mk(2, 50, 512), mk(2, 50, 512)
+    seen = []
+
+    def twice(t):
+        seen.append((t.dtype, tuple(t.shape)))
+        t.mul_(2.0)
+
+    def grads(fn, *params):
+        leaves = [p.clone().requires_grad_(True) for p in params]
+        xx = x.clone().requires_grad_(True)
+        fn(xx, *leaves).backward(dy)
+        return [xx.grad] + [p.grad for p in leaves]
+
+    scale, shift, gate = mk(2, 1, 512, scale=0.2), mk(2, 1, 512, scale=0.2), mk(2, 1, 512, scale=0.5)
+    base = grads(lambda xx, sc, sh: AdaLNModelFunction.apply(xx, sc, sh, 1e-6, 512), scale, shift)
+    red = grads(lambda xx, sc, sh: AdaLNGradReduceFunction.apply(xx, sc, sh, 1e-6, 512, twice), scale, shift)
+    assert seen == [(torch.float32, (2, 2, 512))]
+    assert torch.equal(red[0], base[0]) and torch.equal(red[1], 2 * base[1]) and torch.equal(red[2], 2 * base[2])
+    seen.clear()
+    base = grads(lambda xx, gt: GateResidualFunction.apply(xx, gt, r), gate)
+    red = grads(lambda xx, gt: GateResidualGradReduceFunction.apply(xx, gt, r, twice), gate)
+    assert seen == [(torch.float32, (2, 512))]
+    assert torch.equal(red[0], base[0]) and torch.equal(red[1], 2 * base[1])
+
+
+def test_swap_in_with_a_reduce_hook_on_a_context_parallel_block(monkeypatch):
+    """A block that routes its modulations and gates through *_with_cp_grad_reduce callables
+    (parallel_wan_model.py:18-37), several ranks pretended: with cp_grad_reduce the callables are
+    replaced by fused ops whose parameter gradients pass through the hook, and agree with the
+    reference's hand-written Functions (context_parallel/layers.py:24-53) using the same stand-in for
+    the all-reduce."""
+    from teletron_amd import swap_in as S
+    fake_all_reduce = lambda t: t.mul_(2.0)
+
+    class GateRef(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, gate, residual):
+            ctx.save_for_backward(gate, residual)
+            return x + gate * residual
+
+        @staticmethod
+        def backward(ctx, x_grad):
+            gate, residual = ctx.saved_tensors
+            gate_grad = torch.sum(x_grad * residual, dim=1, keepdim=True)
+            fake_all_reduce(gate_grad)
+            return x_grad, gate_grad, x_grad * gate
+
+    class ModulateRef(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, shift, scale):
+            ctx.save_for_backward(x, scale)
+            return x * (1 + scale) + shift
+
+        @staticmethod
+        def backward(ctx, grad_output):
+            x, scale = ctx.saved_tensors
+            scale_grad = torch.sum(grad_output * x, dim=1, keepdim=True)
+            shift_grad = torch.sum(grad_output, dim=1, keepdim=True)
+            fake_all_reduce(scale_grad)
+            fake_all_reduce(shift_grad)
+            return grad_output * (1 + scale), shift_grad, scale_grad
+
+    class ContextParallelWanDitBlock(nn.Module):
+        def __init__(self, dim):
+            super().__init__()
+            self.norm1 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
+            self.norm2 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
+            self.ffn = nn.Linear(dim, dim)
+            self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
+            self.modulate_with_cp_grad_reduce = lambda x, shift, scale: ModulateRef.apply(x, shift, scale)
+            self.gate_with_cp_grad_reduce = lambda x, gate, residual: GateRef.apply(x, gate, residual)
+
+        def forward(self, x, t_mod):
+            s1, c1, g1, s2, c2, g2 = (self.modulation.to(dtype=t_mod.dtype) + t_mod).chunk(6, dim=1)
+            x = self.gate_with_cp_grad_reduce(x, g1, self.modulate_with_cp_grad_reduce(self.norm1(x), s1, c1))
+            return self.gate_with_cp_grad_reduce(x, g2, self.ffn(self.modulate_with_cp_grad_reduce(self.norm2(x), s2, c2)))
+
+    torch.manual_seed(23)
+    blk = ContextParallelWanDitBlock(512).to(DEV).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(24)
+    mk = lambda *s, scale=1.0: (scale * torch.randn(*s, generator=g)).to(torch.bfloat16).to(DEV)
+    inputs, dy = [mk(2, 64, 512), mk(2, 6, 512, scale=0.2)], mk(2, 64, 512)
+    out_e, gin_e, gp_e = run(blk, inputs, dy)
+    monkeypatch.setattr(S, "_several_ranks", lambda: True)
+    assert S.swap_in(blk)["modulate"] == 0                                       # not told how to reduce: left alone
+    counts = S.swap_in(blk, cp_grad_reduce=fake_all_reduce)
+    assert counts["modulate"] == 1 and counts["gate"] == 1 and counts["layernorm"] == 2, counts
+    out_f, gin_f, gp_f = run(blk, inputs, dy)
+    assert rel(out_f, out_e) < 5e-3
+    for a, b in zip(gin_f, gin_e):
+        assert rel(a, b) < 2e-2
+    worst = max((rel(gp_f[n], gp_e[n]), n) for n in gp_e)
+    assert worst[0] < 2e-2, worst

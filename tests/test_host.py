@@ -180,6 +180,16 @@ def test_swap_in_leaves_context_parallel_callables_alone_with_several_ranks(monk
     assert not hasattr(many.modulate_with_cp_grad_reduce, "__wrapped__")
     assert "forward" not in many.__dict__
 
+    # told how to reduce, swap_in replaces them with several ranks as well (not the whole-block forward)
+    told = make()
+    told.gate = type("ContextParallelGateModule", (nn.Module,), {"forward": lambda self, x, gate, residual: x + gate * residual})()
+    reduce = lambda t: t
+    counts = S.swap_in(told, blocks=True, cp_grad_reduce=reduce)
+    assert counts["modulate"] == 1 and counts["gate"] == 2 and counts["layernorm"] == 2 and counts["block"] == 0, counts
+    assert hasattr(told.modulate_with_cp_grad_reduce, "__wrapped__") and hasattr(told.gate_with_cp_grad_reduce, "__wrapped__")
+    assert told.gate.__dict__["_tt_grad_reduce"] is reduce and "forward" in told.gate.__dict__
+    assert isinstance(told.norm1, S.DeferredLayerNorm) and "forward" not in told.__dict__
+
 
 def test_glue_modules_find_the_library_by_name_not_by_build_path():
     """The pybind modules must record libteletron_op.so by its soname (found through their
