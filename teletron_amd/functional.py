@@ -225,16 +225,19 @@ class GateResidualGradReduceFunction(Function):
 
 
 class ResidualNormFunction(Function):
-    """``apply(x, residual, gate, scale, shift, epsilon, affine) -> (s, y)``: the residual update of
+    """``apply(x, residual, gate, scale, shift, epsilon, affine, grad_reduce=None) -> (s, y)``: the residual update of
     a DiT block and the normalisation that reads it, one kernel each way
     (``teletron/models/wan/wan_model.py:239-241``).  ``s = x + gate * residual`` (``gate`` None:
     ``x + residual``); ``y = LayerNorm(s) * (1 + scale) + shift``, or ``LayerNorm(s) * scale + shift``
     with ``affine`` (scale / shift = weight / bias of ``nn.LayerNorm``).  Backward adds the gradients
-    arriving at ``s`` and at ``y`` in fp32 and rounds once."""
+    arriving at ``s`` and at ``y`` in fp32 and rounds once.  ``grad_reduce`` (sequence-sharded models,
+    see ``AdaLNGradReduceFunction``) is called once, on one fp32 tensor holding the gradients of the
+    modulation inputs: gate, and scale / shift unless ``affine`` (the weight and bias of an
+    ``nn.LayerNorm`` are module parameters, reduced by the model's own parameter hooks)."""
 
     @staticmethod
-    def forward(ctx, x, residual, gate, scale, shift, epsilon, affine):
-        ctx.eps, ctx.affine = float(epsilon), bool(affine)
+    def forward(ctx, x, residual, gate, scale, shift, epsilon, affine, grad_reduce=None):
+        ctx.eps, ctx.affine, ctx.grad_reduce = float(epsilon), bool(affine), grad_reduce
         ctx.set_materialize_grads(False)
         ctx.metas = [None if t is None else (t.shape, t.dtype) for t in (gate, scale, shift)]
         bf = torch.bfloat16
@@ -253,6 +256,16 @@ class ResidualNormFunction(Function):
         dx, dr, dscale, dshift, dgate = ops.residual_norm_backward(
             grad_y.contiguous(), None if grad_s is None else grad_s.contiguous(), s, residual, gate_c, scale_c,
             ctx.eps, ctx.affine)
+        if ctx.grad_reduce is not None:
+            parts = [g for g in ((dgate,) if ctx.affine else (dscale, dshift, dgate)) if g is not None]
+            if parts:
+                packed = torch.stack(parts)              # fp32 [k, n_batches, C]: one exchange
+                ctx.grad_reduce(packed)
+                parts = list(packed.unbind(0))
+                if not ctx.affine:
+                    dscale, dshift = parts[0], parts[1]
+                if dgate is not None:
+                    dgate = parts[-1]
 
         def param_grad(g, meta, needed):
             if not needed or g is None:
@@ -267,25 +280,34 @@ class ResidualNormFunction(Function):
 
         need = ctx.needs_input_grad
         return (dx if need[0] else None, dr if need[1] else None, param_grad(dgate, ctx.metas[0], need[2]),
-                param_grad(dscale, ctx.metas[1], need[3]), param_grad(dshift, ctx.metas[2], need[4]), None, None)
+                param_grad(dscale, ctx.metas[1], need[3]), param_grad(dshift, ctx.metas[2], need[4]), None, None, None)
 
 
-def residual_adaln(x, residual, gate, shift, scale, eps: float = 1e-6):
+def gate_residual(x, gate, residual, grad_reduce=None):
+    """``x + gate * residual``; ``grad_reduce`` as in ``GateResidualGradReduceFunction``."""
+    if grad_reduce is not None:
+        return GateResidualGradReduceFunction.apply(x, gate, residual, grad_reduce)
+    return GateResidualFunction.apply(x, gate, residual)
+
+
+def residual_adaln(x, residual, gate, shift, scale, eps: float = 1e-6, grad_reduce=None):
     """``s = x + gate * residual`` (gate None: ``x + residual``) and
     ``modulate(layer_norm(s), shift, scale)``; returns ``(s, y)``.  Argument order of ``modulate``.
-    Shapes without a fused kernel (rows of at most 256 elements) run the two fused halves."""
+    Shapes without a fused kernel (rows of at most 256 elements) run the two fused halves.
+    ``grad_reduce``: see ``ResidualNormFunction``."""
     if ops.residual_norm_supported(x):
-        return ResidualNormFunction.apply(x, residual, gate, scale, shift, eps, False)
-    s = GateResidualFunction.apply(x, gate, residual) if gate is not None else x + residual
-    return s, adaln_modulate(s, shift, scale, eps)
+        return ResidualNormFunction.apply(x, residual, gate, scale, shift, eps, False, grad_reduce)
+    s = gate_residual(x, gate, residual, grad_reduce) if gate is not None else x + residual
+    return s, adaln_modulate(s, shift, scale, eps, grad_reduce)
 
 
-def residual_layer_norm(x, residual, gate, weight, bias, eps: float = 1e-5):
+def residual_layer_norm(x, residual, gate, weight, bias, eps: float = 1e-5, grad_reduce=None):
     """``s = x + gate * residual`` (gate None: ``x + residual``) and
-    ``F.layer_norm(s, weight, bias)``; returns ``(s, y)``."""
+    ``F.layer_norm(s, weight, bias)``; returns ``(s, y)``.  ``grad_reduce``: see ``ResidualNormFunction``
+    (it reaches the gate gradient only)."""
     if ops.residual_norm_supported(x):
-        return ResidualNormFunction.apply(x, residual, gate, weight, bias, eps, True)
-    s = GateResidualFunction.apply(x, gate, residual) if gate is not None else x + residual
+        return ResidualNormFunction.apply(x, residual, gate, weight, bias, eps, True, grad_reduce)
+    s = gate_residual(x, gate, residual, grad_reduce) if gate is not None else x + residual
     return s, torch.nn.functional.layer_norm(s, (s.shape[-1],), weight, bias, eps)
 
 
@@ -296,8 +318,11 @@ class FusedGate(nn.Module):
         return GateResidualFunction.apply(x, gate, residual)
 
 
-def adaln_modulate(x, shift, scale, eps: float = 1e-6):
-    """``modulate(layer_norm(x), shift, scale)`` in one kernel (argument order of ``modulate``)."""
+def adaln_modulate(x, shift, scale, eps: float = 1e-6, grad_reduce=None):
+    """``modulate(layer_norm(x), shift, scale)`` in one kernel (argument order of ``modulate``);
+    ``grad_reduce`` as in ``AdaLNGradReduceFunction``."""
+    if grad_reduce is not None:
+        return AdaLNGradReduceFunction.apply(x, scale, shift, eps, x.shape[-1], grad_reduce)
     return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
 
 

@@ -50,7 +50,8 @@ their parameter gradients over the context-parallel group
 which is what the plain fused ops return.  While ``torch.distributed`` runs with more than one rank
 these callables are left as they are unless ``swap_in`` is told how to reduce (``cp_grad_reduce``),
 in which case they are replaced by fused ops that pass their fp32 parameter gradients through that
-callable; the whole-block forwards are not installed on context-parallel blocks then.
+callable, and so is the forward of ``ContextParallelWanDitBlock`` (the HunyuanVideo double-stream
+forward is not installed on context-parallel blocks then).
 """
 from __future__ import annotations
 
@@ -66,8 +67,8 @@ import torch.nn.functional as F
 from . import ops
 from .functional import (AdaLNGradReduceFunction, AdaLNModelFunction, GateResidualFunction,
                          GateResidualGradReduceFunction, RMSNormModelFunction, RMSNormRopeFunction,
-                         RMSNormRopeHeadsFunction, adaln_modulate, residual_adaln, residual_layer_norm,
-                         rope_table_from_cos_sin)
+                         RMSNormRopeHeadsFunction, adaln_modulate, gate_residual, residual_adaln,
+                         residual_layer_norm, rope_table_from_cos_sin)
 
 ADALN_NORM_ATTRS = ("norm1", "norm2", "norm", "norm2_context")
 ADALN_OWNER_CLASSES = ("DiTBlock", "ContextParallelWanDitBlock", "Head", "AdaLayerNormZero", "AdaLayerNormZeroSingle",
@@ -254,13 +255,15 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
         return type(self).forward(self, x, context, t_mod, freqs)
     shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
         self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
-    input_x = adaln_modulate(x, shift_msa, scale_msa, self.norm1.eps)
+    # context-parallel block told how to reduce: the gradients of the six modulation chunks pass through it
+    reduce = self.__dict__.get("_tt_grad_reduce")
+    input_x = adaln_modulate(x, shift_msa, scale_msa, self.norm1.eps, reduce)
     attn_output = self.self_attn(input_x, freqs)
     # x = gate(x, gate_msa, attn_output); norm3(x)
-    x, normed = residual_layer_norm(x, attn_output, gate_msa, self.norm3.weight, self.norm3.bias, self.norm3.eps)
+    x, normed = residual_layer_norm(x, attn_output, gate_msa, self.norm3.weight, self.norm3.bias, self.norm3.eps, reduce)
     # x = x + cross_attn(norm3(x), context); modulate(norm2(x), shift_mlp, scale_mlp)
-    x, input_x = residual_adaln(x, self.cross_attn(normed, context), None, shift_mlp, scale_mlp, self.norm2.eps)
-    return GateResidualFunction.apply(x, gate_mlp, self.ffn(input_x))
+    x, input_x = residual_adaln(x, self.cross_attn(normed, context), None, shift_mlp, scale_mlp, self.norm2.eps, reduce)
+    return gate_residual(x, gate_mlp, self.ffn(input_x), reduce)
 
 
 def _projection_dtype(x: torch.Tensor) -> torch.dtype:
@@ -483,10 +486,10 @@ def _is_self_attention(m: nn.Module) -> bool:
             and _is_rmsnorm(getattr(m, "norm_q", None)) and _is_rmsnorm(getattr(m, "norm_k", None)))
 
 
-def _is_dit_block(m: nn.Module) -> bool:
+def _is_dit_block(m: nn.Module, can_reduce: bool = False) -> bool:
     if type(m).__name__ not in BLOCK_CLASSES:
         return False
-    if type(m).__name__ != "DiTBlock" and _several_ranks():
+    if type(m).__name__ != "DiTBlock" and _several_ranks() and not can_reduce:
         return False      # the context-parallel block all-reduces its modulation gradients over the group
     return (all(hasattr(m, a) for a in ("modulation", "self_attn", "cross_attn", "ffn", "norm1", "norm2"))
             and isinstance(getattr(m, "norm3", None), nn.LayerNorm) and m.norm3.elementwise_affine)
@@ -521,7 +524,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
                     module.__dict__["_tt_grad_reduce"] = cp_grad_reduce
                 module.forward = types.MethodType(_fused_gate_forward, module)
                 counts["gate"] += 1
-        if blocks and _is_dit_block(module) and "forward" not in module.__dict__:
+        if blocks and _is_dit_block(module, cp_grad_reduce is not None) and "forward" not in module.__dict__:
+            if type(module).__name__ != "DiTBlock" and cp_grad_reduce is not None:
+                module.__dict__["_tt_grad_reduce"] = cp_grad_reduce
             module.forward = types.MethodType(fused_dit_block_forward, module)
             counts["block"] += 1
         if blocks and adaln and gate and _is_hunyuan_double_block(module) and "forward" not in module.__dict__:

@@ -347,6 +347,41 @@ def test_gradient_reducing_variants_hand_fp32_parameter_gradients_to_the_hook():
     assert torch.equal(red[0], base[0]) and torch.equal(red[1], 2 * base[1])
 
 
+def fake_all_reduce(t):
+    """Stands for the all-reduce over a context-parallel group of two ranks holding the same rows."""
+    t.mul_(2.0)
+
+
+class GateRef(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, gate, residual):
+        ctx.save_for_backward(gate, residual)
+        return x + gate * residual
+
+    @staticmethod
+    def backward(ctx, x_grad):
+        gate, residual = ctx.saved_tensors
+        gate_grad = torch.sum(x_grad * residual, dim=1, keepdim=True)
+        fake_all_reduce(gate_grad)
+        return x_grad, gate_grad, x_grad * gate
+
+
+class ModulateRef(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, shift, scale):
+        ctx.save_for_backward(x, scale)
+        return x * (1 + scale) + shift
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, scale = ctx.saved_tensors
+        scale_grad = torch.sum(grad_output * x, dim=1, keepdim=True)
+        shift_grad = torch.sum(grad_output, dim=1, keepdim=True)
+        fake_all_reduce(scale_grad)
+        fake_all_reduce(shift_grad)
+        return grad_output * (1 + scale), shift_grad, scale_grad
+
+
 def test_swap_in_with_a_reduce_hook_on_a_context_parallel_block(monkeypatch):
     """A block that routes its modulations and gates through *_with_cp_grad_reduce callables
     (parallel_wan_model.py:18-37), several ranks pretended: with cp_grad_reduce the callables are
@@ -354,36 +389,6 @@ def test_swap_in_with_a_reduce_hook_on_a_context_parallel_block(monkeypatch):
     reference's hand-written Functions (context_parallel/layers.py:24-53) using the same stand-in for
     the all-reduce."""
     from teletron_amd import swap_in as S
-    fake_all_reduce = lambda t: t.mul_(2.0)
-
-    class GateRef(torch.autograd.Function):
-        @staticmethod
-        def forward(ctx, x, gate, residual):
-            ctx.save_for_backward(gate, residual)
-            return x + gate * residual
-
-        @staticmethod
-        def backward(ctx, x_grad):
-            gate, residual = ctx.saved_tensors
-            gate_grad = torch.sum(x_grad * residual, dim=1, keepdim=True)
-            fake_all_reduce(gate_grad)
-            return x_grad, gate_grad, x_grad * gate
-
-    class ModulateRef(torch.autograd.Function):
-        @staticmethod
-        def forward(ctx, x, shift, scale):
-            ctx.save_for_backward(x, scale)
-            return x * (1 + scale) + shift
-
-        @staticmethod
-        def backward(ctx, grad_output):
-            x, scale = ctx.saved_tensors
-            scale_grad = torch.sum(grad_output * x, dim=1, keepdim=True)
-            shift_grad = torch.sum(grad_output, dim=1, keepdim=True)
-            fake_all_reduce(scale_grad)
-            fake_all_reduce(shift_grad)
-            return grad_output * (1 + scale), shift_grad, scale_grad
-
     class ContextParallelWanDitBlock(nn.Module):
         def __init__(self, dim):
             super().__init__()
@@ -415,3 +420,45 @@ def test_swap_in_with_a_reduce_hook_on_a_context_parallel_block(monkeypatch):
         assert rel(a, b) < 2e-2
     worst = max((rel(gp_f[n], gp_e[n]), n) for n in gp_e)
     assert worst[0] < 2e-2, worst
+
+
+def test_context_parallel_wan_block_forward_with_a_reduce_hook(monkeypatch):
+    """blocks=True on a block with ContextParallelWanDitBlock's forward (parallel_wan_model.py:18-37;
+    complete sub-modules from wan_standins), several ranks pretended: the fused block forward is
+    installed when swap_in is told how to reduce, and every gradient that the reference's Functions
+    all-reduce (the six modulation chunks) passes through the hook."""
+    import wan_standins as W
+    from teletron_amd import swap_in as S
+
+    class ContextParallelWanDitBlock(W.DiTBlock):
+        def __init__(self, *args):
+            super().__init__(*args)
+            self.modulate_with_cp_grad_reduce = lambda x, shift, scale: ModulateRef.apply(x, shift, scale)
+            self.gate_with_cp_grad_reduce = lambda x, gate, residual: GateRef.apply(x, gate, residual)
+
+        def forward(self, x, context, t_mod, freqs):
+            s1, c1, g1, s2, c2, g2 = (self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
+            x = self.gate_with_cp_grad_reduce(x, g1, self.self_attn(self.modulate_with_cp_grad_reduce(self.norm1(x), s1, c1), freqs))
+            x = x + self.cross_attn(self.norm3(x), context)
+            return self.gate_with_cp_grad_reduce(x, g2, self.ffn(self.modulate_with_cp_grad_reduce(self.norm2(x), s2, c2)))
+
+    c = W.CASE
+    model = W.build_case_model(ContextParallelWanDitBlock, W.Head, (c["dim"], c["num_heads"], c["ffn_dim"], c["eps"]),
+                               (c["dim"], c["out_dim"], c["patch_size"], c["eps"]), c)
+    inputs = W.case_inputs()
+    eager = W.run_case(model, inputs, DEV, torch.bfloat16)
+    monkeypatch.setattr(S, "_several_ranks", lambda: True)
+    first = S.swap_in(model, blocks=True)                                    # not told how to reduce: the blocks and their
+    assert first["block"] == 0 and first["modulate"] == 0 and first["gate"] == 4, first   # CP callables stay (GateModules go)
+    counts = S.swap_in(model, blocks=True, cp_grad_reduce=fake_all_reduce)
+    assert counts["block"] == 2 and counts["modulate"] == 2 and counts["gate"] == 2 and counts["layernorm"] == 4, counts
+    fused = W.run_case(model, inputs, DEV, torch.bfloat16)
+    assert rel(fused[0], eager[0]) < 5e-3
+    for a, b in zip(fused[1], eager[1]):
+        assert rel(a, b) < 2e-2, rel(a, b)
+    # the key bias of the cross attention has a nearly cancelling gradient (6e-2 from the float32 truth in eager
+    # bf16 as well, see test_gpu_wan_vectors.py): it is given 4e-2 here, every other parameter the usual 2e-2
+    errs = {n: rel(fused[2][n], eager[2][n]) for n in eager[2]}
+    worst = max((e, n) for n, e in errs.items() if not n.endswith("cross_attn.k.bias"))
+    assert worst[0] < 2e-2, worst
+    assert max(e for n, e in errs.items() if n.endswith("cross_attn.k.bias")) < 4e-2
