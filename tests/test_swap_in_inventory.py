@@ -285,6 +285,13 @@ def test_context_parallel_assignments_are_recognised(monkeypatch):
     assert counts["gate"] == 2 and counts["modulate"] == 1 and counts["block"] == 1, counts
     assert isinstance(root.m2.norm1, nn.LayerNorm) and isinstance(root.m0.norm1.norm, nn.LayerNorm)
     assert isinstance(root.m0.norm2, S.DeferredLayerNorm)      # inline modulation: row-local, no all-reduce involved
+    # told how to reduce, the assigned callables are replaced with several ranks too; the double-stream block forward
+    # is not (its inline modulation after norm2 is not reduced by the reference, the fused pair would reduce it)
+    root = assigned_model()
+    counts = S.swap_in(root, blocks=True, cp_grad_reduce=lambda t: t)
+    assert counts["gate"] == 2 + 1 + 2 and counts["modulate"] == 3 + 1 and counts["block"] == 2, counts
+    assert "forward" not in root.m0.__dict__ and "forward" in root.m1.__dict__ and "forward" in root.m2.__dict__
+    assert hasattr(root.m0.gate, "__wrapped__") and hasattr(root.m0.norm1.modulate, "__wrapped__")
 
 
 def test_replacement_forwards_keep_the_recorded_signatures():
