@@ -43,6 +43,12 @@ constexpr int kNarrowR = 2;    // loads per lane and tensor in flight, narrow ke
 // forward launches (reference contract 371 -> 358 us), 1-1.5 % at 32, 64 and 256 columns.  Forward
 // and the AdaLN kernels lose with six (128 columns forward 242 -> 269 us, AdaLN backward 359 -> 363 us).
 constexpr int kNarrowRmsBwdR = 6;
+// RMSNorm forward on narrow rows with every lane slot in use: six loads per lane as well.  As fast as
+// two (2,851,200 x 128: 242 us either way; 16 ... 256 columns within 1 %), but with two the time depends
+// on where the output lies relative to the input (period 128 MiB: 243 us over three quarters of it,
+// up to 279 us over the rest), with six it does not (240-244 us at every offset).  Masked widths keep
+// two (96 columns 282 -> 285 us, 200 columns 369 -> 382 us with six).
+constexpr int kNarrowRmsFwdFullR = 6;
 constexpr int kNarrowNW = 4;   // independent waves per workgroup, narrow kernels
 constexpr int kFwdLoadsPerCu = 18;   // target waves x loads-per-lane per CU, forward
 constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
@@ -108,7 +114,7 @@ KernelInfo info_bwd_saved_narrow() {
 }
 template <int KIND, int L, bool FULL>
 KernelInfo info_fwd_narrow() {
-  constexpr int R = kNarrowR, NW = kNarrowNW;
+  constexpr int R = (KIND == kRMS && FULL) ? kNarrowRmsFwdFullR : kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_fwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
 }
 template <int KIND, int L, bool FULL>
