@@ -274,11 +274,24 @@ static void sweep_mix() {
   }
 }
 
-int main() {
+// Optional arguments: offsets in MiB by which the output buffers and the second input buffers are moved
+// inside their (over-sized) allocations.  Bare streams with few loads in flight depend on where their
+// buffers lie relative to one another (period 128 MiB), so a variant should be judged by its best placement.
+int main(int argc, char** argv) {
+  const size_t out_off = (argc > 1 ? strtoul(argv[1], nullptr, 10) : 0) << 20;
+  const size_t in2_off = (argc > 2 ? strtoul(argv[2], nullptr, 10) : 0) << 20;
+  const size_t slack = (size_t)160 << 20;
   for (int i = 0; i < 6; ++i) {
-    CK(hipMalloc(&buf[i], N * 16));
+    const size_t off = i % 3 == 2 ? out_off : (i % 3 == 1 ? in2_off : 0);
+    if (off > slack) { fprintf(stderr, "offset beyond %zu MiB\n", slack >> 20); return 2; }
+    char* p = nullptr;
+    CK(hipMalloc(&p, N * 16 + slack));
+    buf[i] = reinterpret_cast<u32x4*>(p + off);
     CK(hipMemset(buf[i], 0x11 * (i + 1), N * 16));
   }
+  printf("# output buffers moved by %zu MiB, second inputs by %zu MiB; (in - out) mod 128 MiB = %zu, %zu\n", out_off >> 20,
+         in2_off >> 20, (size_t)(((uintptr_t)buf[0] - (uintptr_t)buf[2]) % ((size_t)128 << 20)) >> 20,
+         (size_t)(((uintptr_t)buf[3] - (uintptr_t)buf[5]) % ((size_t)128 << 20)) >> 20);
   CK(hipMalloc(&bad, 8));
   // leave the idle power state before anything is timed
   for (int w = 0; w < 80; ++w) flat<kTwoReads, kStrided, 1, 2, false><<<256, 512>>>(buf[0], buf[1], buf[2], N, 0);
