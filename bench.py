@@ -54,17 +54,11 @@ def parse_args():
                                       "rmsnorm_small,adaln_odd",
                     help="comma list of further workloads reported under 'also'")
     ap.add_argument("--no-eager-gpu", action="store_true", help="skip timing the eager PyTorch expressions on the GPU")
-    ap.add_argument("--block-demo", action="store_true",
-                    help="also time a whole DiT-block stand-in (Wan2.1-1.3B and 14B widths, 32760 tokens) in eager "
-                         "PyTorch and after swap_in(blocks=True)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device copy of one activation tensor (known size) so "
                          "that hardware byte counters collected over this run can be scaled against it")
     ap.add_argument("--no-function-path", action="store_true",
                     help="skip timing the autograd Functions (the path model code calls) at the workload's shape")
-    ap.add_argument("--ceiling-sweep", action="store_true",
-                    help="run teletron_amd/ceiling_sweep (bare read / write / copy / 2r1w streams under every address "
-                         "layout and store path) and print its table instead of the benchmark line")
     return ap.parse_args()
 
 
@@ -355,161 +349,6 @@ def eager_gpu(w, iters=5):
     return (time.perf_counter() - t0) / iters * 1e3
 
 
-def block_demo(dim=1536, heads=12, ffn_dim=8960, seq=32760, ctx_len=512, iters=3):
-    """Whole-block view (--block-demo): a stand-in with the structure of Wan's DiTBlock
-    (teletron/models/wan/wan_model.py:126-244: nn.Linear projections, torch SDPA as the attention
-    core, tanh-GELU FFN) timed forward + backward in eager PyTorch and again after
-    swap_in(blocks=True).  The GEMMs and the attention dominate; this shows what the fused
-    normalisation / residual kernels are worth inside a block."""
-    import torch
-    import torch.nn as nn
-    import torch.nn.functional as F
-    from teletron_amd import swap_in as S
-    dev, bf = "cuda:0", torch.bfloat16
-
-    def rope_apply(x, freqs, n):
-        b, s, c = x.shape
-        xc = torch.view_as_complex(x.to(torch.float64).reshape(b, s, n, -1, 2))
-        return torch.view_as_real(xc * freqs).flatten(2).to(x.dtype)
-
-    class RMSNorm(nn.Module):
-        def __init__(self, d, eps):
-            super().__init__()
-            self.eps, self.weight = eps, nn.Parameter(torch.ones(d))
-
-        def forward(self, x):
-            xf = x.float()
-            return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)).to(x.dtype) * self.weight
-
-    class AttentionModule(nn.Module):
-        def forward(self, q, k, v):
-            b, s, c = q.shape
-            sh = lambda t: t.reshape(b, t.shape[1], heads, -1).transpose(1, 2)
-            return F.scaled_dot_product_attention(sh(q), sh(k), sh(v)).transpose(1, 2).reshape(b, s, c)
-
-    class SelfAttention(nn.Module):
-        def __init__(self, cross=False):
-            super().__init__()
-            self.num_heads, self.cross = heads, cross
-            self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
-            self.norm_q, self.norm_k, self.attn = RMSNorm(dim, 1e-6), RMSNorm(dim, 1e-6), AttentionModule()
-
-        def forward(self, x, other):
-            src = other if self.cross else x
-            q, k, v = self.norm_q(self.q(x)), self.norm_k(self.k(src)), self.v(src)
-            if not self.cross:
-                q, k = rope_apply(q, other, heads), rope_apply(k, other, heads)
-            return self.o(self.attn(q, k, v))
-
-    class CrossAttention(SelfAttention):
-        def __init__(self):
-            super().__init__(cross=True)
-
-    class GateModule(nn.Module):
-        def forward(self, x, gate, residual):
-            return x + gate * residual
-
-    class DiTBlock(nn.Module):
-        def __init__(self):
-            super().__init__()
-            self.self_attn, self.cross_attn = SelfAttention(), CrossAttention()
-            self.norm1 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
-            self.norm2 = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
-            self.norm3 = nn.LayerNorm(dim, eps=1e-6)
-            self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate="tanh"), nn.Linear(ffn_dim, dim))
-            self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
-            self.gate, self.gate2 = GateModule(), GateModule()
-
-        def forward(self, x, context, t_mod, freqs):
-            sh1, sc1, g1, sh2, sc2, g2 = (self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
-            x = self.gate(x, g1, self.self_attn(self.norm1(x) * (1 + sc1) + sh1, freqs))
-            x = x + self.cross_attn(self.norm3(x), context)
-            return self.gate2(x, g2, self.ffn(self.norm2(x) * (1 + sc2) + sh2))
-
-    torch.manual_seed(0)
-    blk = DiTBlock().to(dev).to(bf)
-    x = torch.randn(1, seq, dim, device=dev, dtype=bf, requires_grad=True)
-    ctx, dy = torch.randn(1, ctx_len, dim, device=dev, dtype=bf), torch.randn(1, seq, dim, device=dev, dtype=bf)
-    t_mod = 0.2 * torch.randn(1, 6, dim, device=dev, dtype=bf)
-    ang = torch.randn(seq, dim // heads // 2, dtype=torch.float64)
-    freqs = torch.polar(torch.ones_like(ang), ang).reshape(seq, 1, -1).to(dev)
-
-    def timed():
-        for i in range(2 + iters):
-            if i == 2:
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-            blk(x, ctx, t_mod, freqs).backward(dy)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / iters * 1e3
-
-    eager_ms = timed()
-    out_e = blk(x, ctx, t_mod, freqs).detach()
-    counts = S.swap_in(blk, blocks=True)
-    fused_ms = timed()
-    out_f = blk(x, ctx, t_mod, freqs).detach()
-    diff = float((out_f.double() - out_e.double()).norm() / out_e.double().norm())
-    return {"block": f"DiTBlock stand-in, dim {dim}, {heads} heads, ffn {ffn_dim}, x[1,{seq},{dim}] bf16, context {ctx_len}",
-            "eager_ms": round(eager_ms, 2), "fused_ms": round(fused_ms, 2), "speedup": round(eager_ms / fused_ms, 3),
-            "relative_output_difference": diff, "swapped": counts}
-
-
-def hunyuan_block_demo(kind="single", n_img=16384, n_txt=256, n_blocks=3, heads=24, head_dim=128, iters=4):
-    """Whole-block view for HunyuanVideo (--block-demo): `n_blocks` single- or double-stream blocks in a row, built
-    from the stand-ins the swap-in tests use (tests/hunyuan_standins.py: the call pattern of
-    teletron/models/hunyuan/model.py:64-170,472-583 around nn.Linear and torch SDPA), forward +
-    backward in eager PyTorch, after swap_in() and after swap_in(blocks=True) (fused per-head norm +
-    rotary embedding in the processor, token sequence no longer copied at every re-join)."""
-    import torch
-    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
-    import hunyuan_standins as H
-    from teletron_amd import swap_in as S
-    dev, bf, dim = "cuda:0", torch.bfloat16, heads * head_dim
-
-    def build():
-        torch.manual_seed(0)
-        cls = H.HunyuanVideoSingleTransformerBlock if kind == "single" else H.HunyuanVideoTransformerBlock
-        return torch.nn.ModuleList([cls(heads, head_dim, mlp_ratio=4) for _ in range(n_blocks)]).to(dev).to(bf)
-
-    g = torch.Generator(device=dev).manual_seed(1)
-    rnd = lambda *shape: torch.randn(*shape, device=dev, generator=g)
-    h, e, temb = rnd(1, n_img, dim).to(bf), rnd(1, n_txt, dim).to(bf), rnd(1, dim).to(bf)
-    ang = 3.0 * rnd(n_img, head_dim // 2)
-    rotary = (ang.cos().repeat_interleave(2, 1), ang.sin().repeat_interleave(2, 1))
-    dy = rnd(1, n_img + n_txt, dim).to(bf)
-
-    def step(m, hh, ee):
-        for blk in m:
-            hh, ee = blk(hh, ee, temb, None, rotary)
-        out = torch.cat([hh, ee], 1)
-        out.backward(dy)
-        return out.detach()
-
-    def timed(m):
-        hh, ee = h.clone().requires_grad_(True), e.clone().requires_grad_(True)
-        for i in range(2 + iters):
-            if i == 2:
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-            out = step(m, hh, ee)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / iters * 1e3, out
-
-    eager_ms, out_e = timed(build())
-    m = build()
-    S.swap_in(m)
-    swapped_ms, _ = timed(m)
-    m = build()
-    counts = S.swap_in(m, blocks=True)
-    blocks_ms, out_f = timed(m)
-    diff = float((out_f.double() - out_e.double()).norm() / out_e.double().norm())
-    name = "HunyuanVideoSingleTransformerBlock" if kind == "single" else "HunyuanVideoTransformerBlock"
-    return {"block": f"{n_blocks} {name} stand-ins, dim {dim}, {heads} heads, "
-                     f"{n_img} latent + {n_txt} text tokens, bf16",
-            "eager_ms": round(eager_ms, 2), "swap_in_ms": round(swapped_ms, 2), "swap_in_blocks_ms": round(blocks_ms, 2),
-            "speedup": round(eager_ms / blocks_ms, 3), "relative_output_difference": diff, "swapped": counts}
-
-
 def function_path(w, cabi_ms, iters=50):
     """The path model code calls: AdaLNModelFunction / RMSNormModelFunction apply + backward on
     tensors of the workload's shape, parameters as the model passes them ([B, 1, C] modulation,
@@ -621,13 +460,6 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HIP kernels have no CPU fallback.", file=sys.stderr)
         return 2
-    if args.ceiling_sweep:
-        import subprocess
-        exe = os.path.join(REPO_ROOT, "teletron_amd", "ceiling_sweep")
-        if not os.path.exists(exe):
-            print(f"{exe} is missing: run `python -m teletron_amd.build` first.", file=sys.stderr)
-            return 2
-        return subprocess.run([exe]).returncode
     w = WORKLOADS[args.workload]
     r = measure(w, args.steps, args.warmup, ceiling=True)
     mt = MEASURED_TRAFFIC_BYTES.get(w.name)
@@ -687,9 +519,6 @@ def main():
                 also[name]["speedup_vs_eager_gpu"] = round(ms / ra["ms_per_step"], 2)
     if also:
         out["also"] = also
-    if args.block_demo:
-        out["block_demo"] = [block_demo(1536, 12, 8960), block_demo(5120, 40, 13824), hunyuan_block_demo("single"),
-                             hunyuan_block_demo("double", n_blocks=2)]
     if args.calibrate_copy:
         src = torch.empty(w.elements, dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
         dst = torch.empty_like(src)

@@ -74,20 +74,6 @@ def build_library(force: bool = True, defines=(), jobs: int = 8, verbose: bool =
     return LIB_PATH
 
 
-SWEEP_PATH = PKG_DIR / "ceiling_sweep"
-
-
-def build_ceiling_sweep(verbose: bool = True) -> Path:
-    """Compile the stand-alone stream-ceiling measurement program (csrc/ceiling_sweep.hip), which
-    ``bench.py --ceiling-sweep`` runs.  It does not link against the library."""
-    if verbose:
-        print("[teletron_amd.build] hipcc ceiling_sweep.hip", flush=True)
-    _run([hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-o", str(SWEEP_PATH),
-          str(CSRC / "ceiling_sweep.hip")])
-    return SWEEP_PATH
-
-
 TORCH_EXT_MODULES = ["fused_adaln", "fused_rmsnorm"]
 
 
@@ -143,7 +129,6 @@ def main(argv=None) -> int:
     build_library(force=args.force or bool(args.define), defines=args.define, jobs=args.jobs)
     if not args.no_torch_ext:
         build_torch_extensions(force=args.force)
-    build_ceiling_sweep()
     return 0
 
 
