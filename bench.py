@@ -49,7 +49,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target wall time of the CPU leg")
     ap.add_argument("--also", default="rmsnorm_wan14b_qk,rmsnorm_hunyuan_head,adaln_wan1p3b_batched,"
-                                      "adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
+                                      "adaln_hunyuan,adaln_hunyuan_reference_contract,rmsnorm_hunyuan_head_reference_contract,"
                                       "residual_adaln_wan14b,gated_residual_layernorm_wan14b,rmsnorm_rope_hunyuan_head,"
                                       "rmsnorm_small,adaln_odd",
                     help="comma list of further workloads reported under 'also'")
@@ -211,9 +211,11 @@ class GpuWorkload:
         self.cabi.call("tt_reduce_partials", self.g0.data_ptr(), self.g1.data_ptr() if self.n_acc == 2 else None,
                        self.ws.data_ptr(), self.nb, self.n_partials.value, self.n_acc, self.cols, self.stream)
 
-    def stream_ceiling(self, iters=12):
+    def stream_ceiling(self, iters=12, mix_only=None):
         """Bare streams over this workload's own buffers (no arithmetic, same load/store policy):
-        GB/s of one-read-one-write (x -> y) and two-reads-one-write (x ^ dy -> dx) traffic."""
+        GB/s of one-read-one-write (x -> y), two-reads-one-write (x ^ dy -> dx), read-only and
+        write-only traffic; `mix_only="1r2w"`: only one-read-two-writes (x -> y, x_norm), the traffic
+        of the reference contract's AdaLN forward."""
         torch = self.torch
         nbytes = self.rows * self.cols * 2
 
@@ -225,14 +227,19 @@ class GpuWorkload:
                 a = None if mix == "write" else s["x"].data_ptr()
                 b = s["dy"].data_ptr() if mix == "2r1w" else None
                 e[0].record()
-                self.cabi.call("tt_stream_probe", out, a, b, nbytes, self.stream)
+                if mix == "1r2w":
+                    self.cabi.call("tt_stream_probe_two_outputs", s["y"].data_ptr(), s["x_norm"].data_ptr(), a, nbytes, self.stream)
+                else:
+                    self.cabi.call("tt_stream_probe", out, a, b, nbytes, self.stream)
                 e[1].record()
             torch.cuda.synchronize()
             t = statistics.median(e[0].elapsed_time(e[1]) for e in ev[3:]) * 1e-3
-            return {"read": 1, "write": 1, "copy": 2, "2r1w": 3}[mix] * nbytes / t / 1e9
+            return {"read": 1, "write": 1, "copy": 2, "2r1w": 3, "1r2w": 3}[mix] * nbytes / t / 1e9
 
         # the bare copy depends on where the two buffers lie relative to one another (period 128 MiB:
         # fast over one half of it, up to 25 % slower over the other); say where these lie
+        if mix_only:
+            return {mix_only: timed(mix_only)}
         placement = [round(((s["x"].data_ptr() - s["y"].data_ptr()) % (128 << 20)) / 2 ** 20, 1) for s in self.sets]
         return {"copy": timed("copy"), "two_reads_one_write": timed("2r1w"),
                 "read_only": timed("read"), "write_only": timed("write"), "copy_in_minus_out_mod_128MiB": placement}
@@ -349,24 +356,37 @@ def eager_gpu(w, iters=5):
     return (time.perf_counter() - t0) / iters * 1e3
 
 
-def function_path(w, cabi_ms, iters=50):
-    """The path model code calls: AdaLNModelFunction / RMSNormModelFunction apply + backward on
-    tensors of the workload's shape, parameters as the model passes them ([B, 1, C] modulation,
-    [C] weight), two alternating input sets.  Wall milliseconds per forward+backward and the
-    ratio to the C-ABI step of the same workload."""
+def function_path(w, cabi_ms, kind="plain", iters=50):
+    """The path model code calls: the autograd Function's apply + backward on tensors of the
+    workload's shape, parameters as the model passes them ([B, 1, C] modulation, [C] weight), two
+    alternating input sets.  Per-head workloads ([1, S, H, D] in memory) are handed over as
+    HunyuanVideo does (teletron/models/hunyuan/model.py:87-95): the [B, H, S, D] transposed view,
+    and the incoming gradient in that same layout.  kind "rope_heads": RMSNormRopeHeadsFunction on
+    that view.  Wall milliseconds per forward+backward and the ratio to the C-ABI step of the
+    same workload."""
     import torch
-    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction
+    from teletron_amd import AdaLNModelFunction, RMSNormModelFunction, RMSNormRopeHeadsFunction
     dev, bf = "cuda:0", torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(2)
     rnd = lambda *shape, scale=1.0, offset=0.0: (offset + scale * torch.randn(*shape, generator=g, device=dev)).to(bf)
-    xs = [rnd(*w.shape).requires_grad_(True) for _ in range(2)]
-    dys = [rnd(*w.shape) for _ in range(2)]
+    per_head = len(w.shape) == 4
+    view = (lambda t: t.transpose(1, 2)) if per_head else (lambda t: t)
+    bufs = [rnd(*w.shape) for _ in range(2)]
+    xs = [view(t).requires_grad_(True) for t in bufs]      # leaf tensors in the layout the model holds
+    dys = [view(rnd(*w.shape)) for _ in range(2)]
     if w.op == "adaln":
         scale = rnd(*w.param_shape, scale=0.1).requires_grad_(True)
         shift = rnd(*w.param_shape, scale=0.1).requires_grad_(True)
         params = [scale, shift]
         op = lambda i: AdaLNModelFunction.apply(xs[i], scale, shift, w.eps, w.cols)
         name = "AdaLNModelFunction"
+    elif kind == "rope_heads":
+        weight = rnd(*w.param_shape, scale=0.1, offset=1.0).requires_grad_(True)
+        ang = 3.0 * torch.randn(w.shape[1], w.cols // 2, generator=g, device=dev, dtype=torch.float32)
+        table = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()
+        params = [weight]
+        op = lambda i: RMSNormRopeHeadsFunction.apply(xs[i], weight, table, w.eps)
+        name = "RMSNormRopeHeadsFunction"
     else:
         weight = rnd(*w.param_shape, scale=0.1, offset=1.0).requires_grad_(True)
         params = [weight]
@@ -386,7 +406,8 @@ def function_path(w, cabi_ms, iters=50):
         fn(i & 1)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / iters * 1e3
-    return {"function": name, "ms_per_step": round(ms, 4), "ratio_to_c_abi_step": round(ms / cabi_ms, 4),
+    return {"function": name, "workload": w.name, "input": "x" + str(list(xs[0].shape)) + (" (transposed view)" if per_head else ""),
+            "ms_per_step": round(ms, 4), "c_abi_ms_per_step": round(cabi_ms, 4), "ratio_to_c_abi_step": round(ms / cabi_ms, 4),
             "note": "apply + backward through torch.autograd, .grad cleared before each step"}
 
 
@@ -445,6 +466,8 @@ def measure(w, steps, warmup, ceiling=False):
     }
     if ceiling:
         res["ceiling"] = g.stream_ceiling()
+    if g.ref and w.op == "adaln":
+        res["ceiling_1r2w"] = g.stream_ceiling(mix_only="1r2w")["1r2w"]
     del g   # the caching allocator keeps the blocks: later workloads reuse them instead of fresh driver memory
     return res
 
@@ -494,6 +517,8 @@ def main():
         "forward_frac_of_copy": round(r["fwd_gbps"] / c["copy"], 4),
         "backward_frac_of_two_reads_one_write": round(r["bwd_gbps"] / c["two_reads_one_write"], 4),
         "copy_in_minus_out_mod_128MiB": c["copy_in_minus_out_mod_128MiB"],
+        **({"one_read_two_writes": round(r["ceiling_1r2w"], 1),
+            "forward_frac_of_one_read_two_writes": round(r["fwd_gbps"] / r["ceiling_1r2w"], 4)} if "ceiling_1r2w" in r else {}),
         "note": "tt_stream_probe: no-arithmetic kernels with the same load/store policy on the same buffers; the bare "
                 "copy is up to 25 % slower when (x - y) mod 128 MiB falls in about [104, 128) or [0, 38) MiB, the "
                 "normalisation kernels are not"}
@@ -509,6 +534,11 @@ def main():
         also[name] = {"value": round(ra["gbps"], 1), "unit": "GB/s", "pct_of_peak": round(100 * ra["gbps"] / HBM_PEAK_GBPS, 2),
                       "ms_per_step": round(ra["ms_per_step"], 4), "forward_us": round(ra["fwd_us"], 2),
                       "backward_streaming_us": round(ra["bwd_us"], 2), "reduce_partials_us": round(ra["reduce_us"], 2)}
+        if "ceiling_1r2w" in ra:
+            # the forward of this contract also stores x_norm: one read, two writes
+            also[name]["stream_ceiling_one_read_two_writes"] = round(ra["ceiling_1r2w"], 1)
+            also[name]["forward_gbps"] = round(ra["fwd_gbps"], 1)
+            also[name]["forward_frac_of_one_read_two_writes"] = round(ra["fwd_gbps"] / ra["ceiling_1r2w"], 4)
         if wa.elements * 2 < CACHE_RESIDENT_BYTES:
             # every tensor fits the 256 MB Infinity Cache: reported, not an HBM figure
             also[name]["cache_resident"] = True
@@ -528,6 +558,14 @@ def main():
         out["calibration_copy_bytes"] = src.numel() * 2
     if not args.no_function_path and w.op in ("adaln", "rmsnorm") and w.contract == "native":
         out["function_path"] = function_path(w, r["ms_per_step"])
+        # the other paths the models call, where the C-ABI step of the same workload was measured above
+        more = []
+        for name, kind in (("rmsnorm_wan14b_qk", "plain"), ("rmsnorm_hunyuan_head", "plain"),
+                           ("rmsnorm_rope_hunyuan_head", "rope_heads")):
+            if name in also:
+                more.append(function_path(WORKLOADS[name], also[name]["ms_per_step"], kind, iters=30))
+        if more:
+            out["function_path_also"] = more
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
         small = WORKLOADS["rmsnorm_small"]

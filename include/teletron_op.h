@@ -263,6 +263,11 @@ TT_API size_t tt_residual_norm_backward_workspace_bytes(int64_t rows, int64_t co
  * out and a, is TT_ERR_INVALID_ARGUMENT. */
 TT_API int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void* stream);
 
+/* The same for one read and two writes, the traffic of tt_launch_adaln_forward (which stores
+ * x_norm next to the output): out0[i] = a[i], out1[i] = ~a[i].  No counterpart in the reference.
+ * All three pointers are required (TT_ERR_INVALID_ARGUMENT); sizes and alignment as above. */
+TT_API int tt_stream_probe_two_outputs(void* out0, void* out1, const void* a, size_t bytes, void* stream);
+
 /* ------------------------------------------------------------------ reference-compatible contract
  * Argument for argument the launchers the reference's pybind glue calls, plus a trailing
  * stream (the reference launches on the legacy default stream) and, for backward, the

@@ -19,7 +19,7 @@ CSRC = PKG_DIR / "csrc"
 OBJ_DIR = CSRC / "build"
 LIB_PATH = PKG_DIR / "libteletron_op.so"
 
-HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_bwd.hip", "adaln_bwd_saved.hip",
+HIP_SOURCES = ["capi.hip", "adaln_fwd.hip", "adaln_fwd_xnorm.hip", "adaln_bwd.hip", "adaln_bwd_saved.hip",
                "rms_fwd.hip", "rms_bwd.hip", "rms_bwd_saved.hip", "rms_rope.hip", "gate.hip",
                "resnorm_plain.hip", "resnorm_gated.hip"]
 

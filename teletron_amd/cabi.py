@@ -77,6 +77,7 @@ PROTOTYPES = {
                                           c_void_p, c_size_t, c_int64, c_int64, c_int64, c_float, c_void_p]),
     "tt_residual_norm_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
     "tt_stream_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "tt_stream_probe_two_outputs": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tt_launch_adaln_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int64, c_double, c_void_p, c_void_p]),
     "tt_launch_adaln_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -107,7 +107,7 @@ struct Plan {
   int packs = 0;
 };
 
-enum Dir { kFwd, kBwd, kBwdSaved };
+enum Dir { kFwd, kBwd, kBwdSaved, kFwdXn };   // kFwdXn: AdaLN forward that also stores x_norm
 constexpr int kGateKind = 2;   // third op family next to kAdaLN / kRMS
 
 // Upper bound on workgroups per batch used by any plan: what the workspace is sized for.
@@ -128,11 +128,14 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   const bool full = (slots == packs);
   KernelInfo k;
   if (res) {
-    if (narrow || kind != kAdaLN || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
+    if (narrow || kind != kAdaLN || dir == kBwdSaved || dir == kFwdXn) return TT_ERR_UNSUPPORTED;
     k = res == 2 ? resnorm_gated_kernel(dir == kBwd, idx, full) : resnorm_plain_kernel(dir == kBwd, idx, full);
   } else if (rope) {
-    if (kind != kRMS || dir == kBwdSaved) return TT_ERR_UNSUPPORTED;
+    if (kind != kRMS || dir == kBwdSaved || dir == kFwdXn) return TT_ERR_UNSUPPORTED;
     k = rms_rope_kernel(narrow, dir == kBwd, idx, full, rope_heads);
+  } else if (dir == kFwdXn) {
+    if (kind != kAdaLN) return TT_ERR_UNSUPPORTED;
+    k = adaln_fwd_xnorm_kernel(narrow, idx, full);
   } else if (kind == kAdaLN)
     k = dir == kFwd ? adaln_fwd_kernel(narrow, idx, full)
       : dir == kBwd ? adaln_bwd_kernel(narrow, idx, full) : adaln_bwd_saved_kernel(narrow, idx, full);
@@ -158,7 +161,8 @@ int make_plan(int kind, Dir dir, int64_t rows, int64_t cols, int64_t rows_per_ba
   if (!cache_resident) {
     const int per_wg = (k.threads / kWave) * k.lane_loads;
     // two streamed inputs (backward kernels, both gate kernels) or one (normalisation forward)
-    const int target = (dir == kFwd && kind != kGateKind && !res) ? kFwdLoadsPerCu : kBwdLoadsPerCu;
+    const int target = dir == kFwdXn ? kFwdXnLoadsPerCu
+                     : (dir == kFwd && kind != kGateKind && !res) ? kFwdLoadsPerCu : kBwdLoadsPerCu;
     int want = (2 * target + per_wg) / (2 * per_wg);
     if (want < 1) want = 1;
     if (want < per_cu) per_cu = want;
@@ -338,7 +342,9 @@ int forward(int kind, void* y, const void* x, const void* p0, const void* p1, fl
     return forward_generic(kind, y, x, p0, p1, mean, rstd, x_norm, rows, cols, rows_per_batch, eps, stream);
   }
   Plan p;
-  int rc = make_plan(kind, kFwd, rows, cols, rows_per_batch, &p, rope != nullptr, 0, rope ? rope->heads : 0);
+  if (x_norm && (kind != kAdaLN || rope)) return TT_ERR_UNSUPPORTED;
+  int rc = make_plan(kind, x_norm ? kFwdXn : kFwd, rows, cols, rows_per_batch, &p, rope != nullptr, 0,
+                     rope ? rope->heads : 0);
   if (rc != TT_OK) return rc;
   FwdArgs a;
   a.freqs = rope ? rope->freqs : nullptr; a.seq_len = rope ? rope->seq_len : 1; a.head_dim = rope ? (int)rope->head_dim : 8;
@@ -684,6 +690,24 @@ int tt_stream_probe(void* out, const void* a, const void* b, size_t bytes, void*
   else if (!a) hipLaunchKernelGGL((stream_probe<kProbeWrite, 1>), grid, dim3(threads), 0, s, out, a, b, n);
   else if (b)  hipLaunchKernelGGL((stream_probe<kProbeXor, 1>), grid, dim3(threads), 0, s, out, a, b, n);
   else         hipLaunchKernelGGL((stream_probe<kProbeCopy, 2>), grid, dim3(threads), 0, s, out, a, b, n);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TT_OK : hip_fail(e);
+}
+
+int tt_stream_probe_two_outputs(void* out0, void* out1, const void* a, size_t bytes, void* stream) {
+  if (bytes == 0) return TT_OK;
+  if (!out0 || !out1 || !a) return TT_ERR_INVALID_ARGUMENT;
+  if (bytes % 16 != 0 || !aligned16(out0) || !aligned16(out1) || !aligned16(a)) return TT_ERR_UNSUPPORTED;
+  int cus = 0;
+  const int rc = current_device_cus(&cus);
+  if (rc != TT_OK) return rc;
+  // four waves per CU with four packs per lane in flight streamed this mix fastest on MI355X
+  constexpr int kThreads = 256, kU = 4;
+  const size_t n = bytes / 16;
+  const size_t tiles = (n + kThreads * kU - 1) / (kThreads * kU);
+  const dim3 grid((unsigned)(tiles < (size_t)cus ? tiles : (size_t)cus));
+  hipLaunchKernelGGL((stream_probe_two_outputs<kU>), grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                     out0, out1, a, n);
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? TT_OK : hip_fail(e);
 }

@@ -32,6 +32,14 @@ __device__ __forceinline__ void store_stream(void* base, size_t elem_off, u32x4 
   // write of those registers (the data is read after issue).  Four are spent on each side.
   asm volatile("s_nop 3\n\tglobal_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 3" ::"v"(p), "v"(v) : "memory");
 }
+// Two stores of one lane to the same element offset of two tensors (an output and a second
+// saved copy): one asm block, so the pair pays the hazard padding once.
+__device__ __forceinline__ void store_stream2(void* base0, void* base1, size_t elem_off, u32x4 v0, u32x4 v1) {
+  u32x4* p0 = reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base0) + elem_off);
+  u32x4* p1 = reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base1) + elem_off);
+  asm volatile("s_nop 3\n\tglobal_store_dwordx4 %0, %2, off sc0 sc1 nt\n\t"
+               "global_store_dwordx4 %1, %3, off sc0 sc1 nt\n\ts_nop 3" ::"v"(p0), "v"(p1), "v"(v0), "v"(v1) : "memory");
+}
 __device__ __forceinline__ u32x4 load_cached(const void* base, size_t elem_off) {
   return *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + elem_off);
 }

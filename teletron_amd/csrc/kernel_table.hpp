@@ -52,6 +52,7 @@ constexpr int kNarrowRmsFwdFullR = 6;
 constexpr int kNarrowNW = 4;   // independent waves per workgroup, narrow kernels
 constexpr int kFwdLoadsPerCu = 18;   // target waves x loads-per-lane per CU, forward
 constexpr int kBwdLoadsPerCu = 12;   // same, backward (per input tensor)
+constexpr int kFwdXnLoadsPerCu = 12; // same, AdaLN forward that also stores x_norm (see fwd_xn_wide_Q)
 
 constexpr int fwd_wide_R(int W, int P) { return 1; }   // two rows per tile: 1-3 % slower at every width
 constexpr int bwd_wide_R(int W, int P) { return 1; }
@@ -121,6 +122,43 @@ template <int KIND, int L, bool FULL>
 KernelInfo info_bwd_narrow() {
   constexpr int R = KIND == kRMS ? kNarrowRmsBwdR : kNarrowR, NW = kNarrowNW;
   return {reinterpret_cast<const void*>(&norm_bwd_narrow<KIND, L, R, NW, FULL>), 64 * NW, NW * R * (64 / L), R};
+}
+
+// AdaLN forward that also stores x_norm (the reference's forward contract): one read and two
+// write streams.  Bare streams of that mix (no arithmetic) reach 5.7-5.9 TB/s on MI355X (370-385 us
+// for the 2.19 GB of 118800 x 3072), and like writes on their own they go fastest with FEW requests
+// in flight: about 12 loads per lane column of a CU (kFwdXnLoadsPerCu), not the 18-20 of the
+// one-output forward.  One row group per workgroup and several independent workgroups per CU:
+// barrier-coupled row groups are 1 % faster at best (118800 x 3072: 379-383 us against 384-390) but
+// 5-8 % slower (400-413 us) over a quarter of the possible placements of the two outputs relative to
+// the input (period 128 MiB); independent workgroups stay at 384-393 us at every placement.
+// Measured with this rule: 75600 x 5120 416 us, 131040 x 1536 213 us, 150000 x 2048 323 us.
+constexpr int fwd_xn_wide_Q(int W, int P) { return 1; }
+template <int W, int P, bool FULL>
+KernelInfo info_fwd_xn_wide() {
+  constexpr int R = fwd_wide_R(W, P), Q = fwd_xn_wide_Q(W, P);
+  return {reinterpret_cast<const void*>(&norm_fwd_wide<kAdaLN, W, P, R, Q, FULL, false, true>), 64 * W * Q, Q * R, P * R};
+}
+template <int L, bool FULL>
+KernelInfo info_fwd_xn_narrow() {
+  constexpr int R = kNarrowR, NW = kNarrowNW;
+  return {reinterpret_cast<const void*>(&norm_fwd_narrow<kAdaLN, L, R, NW, FULL, 0, true>), 64 * NW, NW * R * (64 / L), R};
+}
+inline KernelInfo lookup_fwd_xn(bool narrow, int idx, bool full) {
+  if (narrow) {
+    switch (idx) {
+#define X(i, L) case i: return full ? info_fwd_xn_narrow<L, true>() : info_fwd_xn_narrow<L, false>();
+      TT_NARROW_LIST(X)
+#undef X
+    }
+  } else {
+    switch (idx) {
+#define X(i, W, P) case i: return full ? info_fwd_xn_wide<W, P, true>() : info_fwd_xn_wide<W, P, false>();
+      TT_WIDE_LIST(X)
+#undef X
+    }
+  }
+  return {nullptr, 0, 0, 0};
 }
 
 template <int KIND>
@@ -309,9 +347,10 @@ KernelInfo lookup_bwd_saved(bool narrow, int idx, bool full) {
   return {nullptr, 0, 0, 0};
 }
 
-// Defined one per translation unit (adaln_fwd.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, rms_rope.hip, gate.hip,
+// Defined one per translation unit (adaln_fwd.hip, adaln_fwd_xnorm.hip, adaln_bwd.hip, adaln_bwd_saved.hip, rms_fwd.hip, rms_bwd.hip, rms_bwd_saved.hip, rms_rope.hip, gate.hip,
 // resnorm_plain.hip, resnorm_gated.hip).
 KernelInfo adaln_fwd_kernel(bool narrow, int idx, bool full);
+KernelInfo adaln_fwd_xnorm_kernel(bool narrow, int idx, bool full);
 KernelInfo adaln_bwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_fwd_kernel(bool narrow, int idx, bool full);
 KernelInfo rms_bwd_kernel(bool narrow, int idx, bool full);

@@ -34,7 +34,7 @@ struct FwdArgs {
   const void* p1;   // AdaLN: shift [B, C];  RMSNorm: unused
   float* mean;      // optional [rows]
   float* rstd;      // optional [rows]
-  void* x_norm;     // optional [rows, cols] bf16: the normalised input before modulation (AdaLN)
+  void* x_norm;     // [rows, cols] bf16: the normalised input before modulation (XN kernels only)
   int64_t rows_per_batch;
   int64_t n_tiles;  // tiles per batch
   int cols;
@@ -118,10 +118,12 @@ __device__ __forceinline__ void rowgroup_allsum(float (&v)[NV], float* buf, int 
 }
 
 // ============================================================================ wide forward
-template <int KIND, int W, int P, int R, int Q, bool FULL, bool ROPE = false>
+// XN: also store the normalised input before modulation (a.x_norm), paired with the y store.
+template <int KIND, int W, int P, int R, int Q, bool FULL, bool ROPE = false, bool XN = false>
 __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
   static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
+  static_assert(!XN || ADALN, "x_norm is an output of the AdaLN forward only");
   __shared__ float red[2][Q][W * R];
 
   const int lane = threadIdx.x & 63;
@@ -284,8 +286,8 @@ __global__ __launch_bounds__(64 * W * Q) void norm_fwd_wide(const FwdArgs a) {
               fc[4] = f1[0]; fc[5] = f1[1]; fc[6] = f1[2]; fc[7] = f1[3];
               rope_rotate(o, fc);
             }
-            store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
-            if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col[p]), pack8(n));
+            if constexpr (XN) store_stream2(a.y, a.x_norm, (size_t)(row * C + col[p]), pack8(o), pack8(n));
+            else              store_stream(a.y, (size_t)(row * C + col[p]), pack8(o));
           }
         }
         if (w == 0 && lane == 0) {
@@ -551,10 +553,11 @@ struct RowPos {
 // ROPE: 0 none; 1 every row looks up its own position; 2 the R * 64/L rows a wave takes per tile
 // are exactly the heads of ONE token (the caller guarantees rows_per_pos == R * 64/L), so a lane
 // loads its (cos, sin) entries once per tile instead of once per row.
-template <int KIND, int L, int R, int NW, bool FULL, int ROPE = 0>
+template <int KIND, int L, int R, int NW, bool FULL, int ROPE = 0, bool XN = false>   // XN as in norm_fwd_wide
 __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
   constexpr bool ADALN = (KIND == kAdaLN);
   static_assert(!ROPE || KIND == kRMS, "rotary embedding is fused behind RMSNorm only");
+  static_assert(!XN || ADALN, "x_norm is an output of the AdaLN forward only");
   constexpr int NF = ROPE == 1 ? R : 1;   // table entries held per lane
   constexpr int RPW = 64 / L;
   const int lane = threadIdx.x & 63;
@@ -662,8 +665,8 @@ __global__ __launch_bounds__(64 * NW) void norm_fwd_narrow(const FwdArgs a) {
           o[j] = ADALN ? fmaf(xh, g[j], sh[j]) : xh * g[j];
         }
         if constexpr (ROPE) rope_rotate(o, fc[ROPE == 1 ? r : 0]);
-        store_stream(a.y, (size_t)(row * C + col), pack8(o));
-        if (a.x_norm) store_stream(a.x_norm, (size_t)(row * C + col), pack8(n));
+        if constexpr (XN) store_stream2(a.y, a.x_norm, (size_t)(row * C + col), pack8(o), pack8(n));
+        else              store_stream(a.y, (size_t)(row * C + col), pack8(o));
         if (pi == 0) {
           if (ADALN && a.mean) a.mean[row] = mean;
           if (a.rstd) a.rstd[row] = rstd;

@@ -43,4 +43,42 @@ __global__ void __launch_bounds__(kProbeMaxThreads) stream_probe(void* __restric
   }
 }
 
+// One read, two writes: out0[i] = a[i], out1[i] = ~a[i] (the traffic of a forward that also saves
+// a second tensor).  Persistent tile loop with the next tile prefetched, U packs per lane; a tile's
+// stores go to out0 first, then to out1.
+template <int U>
+__global__ void __launch_bounds__(kProbeMaxThreads) stream_probe_two_outputs(void* __restrict__ out0, void* __restrict__ out1,
+                                                                         const void* __restrict__ a, size_t n) {
+  const size_t T = blockDim.x, tile = T * U;
+  const size_t n_tiles = (n + tile - 1) / tile;
+  u32x4 raw[U];
+  auto fetch = [&](size_t t) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t j = t * tile + u * T + threadIdx.x;
+      raw[u] = u32x4{0, 0, 0, 0};
+      if (j < n) raw[u] = load_stream(a, j * kPack);
+    }
+  };
+  size_t t = blockIdx.x;
+  if (t < n_tiles) fetch(t);
+  for (; t < n_tiles; t += gridDim.x) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = raw[u];
+    if (t + gridDim.x < n_tiles) fetch(t + gridDim.x);
+    __syncthreads();   // lock-step only
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t j = t * tile + u * T + threadIdx.x;
+      if (j < n) store_stream(out0, j * kPack, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t j = t * tile + u * T + threadIdx.x;
+      if (j < n) store_stream(out1, j * kPack, ~v[u]);
+    }
+  }
+}
+
 }  // namespace tt

@@ -82,6 +82,8 @@ WORKLOADS: Dict[str, Workload] = {w.name: w for w in [
     Workload("adaln_odd", "adaln", (3, 5000, 1000), (3, 1, 1000), note="125 packs per row: ragged wave tail"),
     Workload("rmsnorm_rope_wan14b", "rope", (1, 75600, 5120), (5120,), head_dim=128,
              note="Wan2.1-14B QK-norm + rotary embedding, 40 heads of 128"),
+    Workload("adaln_hunyuan", "adaln", (1, 118800, 3072), (1, 1, 3072),
+             note="HunyuanVideo AdaLN sites: the one width the reference kernel supports, native contract"),
     Workload("adaln_hunyuan_reference_contract", "adaln", (1, 118800, 3072), (3072,), contract="reference",
              note="the reference's own AdaLN width, through its launcher signatures"),
     Workload("rmsnorm_hunyuan_head_reference_contract", "rmsnorm", (1, 118800, 24, 128), (128,), contract="reference",

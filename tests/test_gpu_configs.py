@@ -137,6 +137,12 @@ def test_adaln_wan14b_full_size():
     _adaln_full_size("adaln_wan14b", 4096)
 
 
+def test_adaln_hunyuan_full_size():
+    # native contract at the only width the reference kernel supports (adaln_forward.cu:122), at the
+    # HunyuanVideo sequence length: hunyuan/model.py:452-502 call sites
+    _adaln_full_size("adaln_hunyuan", 4096)
+
+
 def test_adaln_batched_full_size():
     _adaln_full_size("adaln_wan1p3b_batched", 8192)
 

@@ -39,6 +39,22 @@ def test_stream_probe_write_only_and_read_only(n_packs):
     assert torch.equal(out, before)
 
 
+@pytest.mark.parametrize("n_packs", [1, 255, 1024, 1025, 256 * 4 * 256 + 77, 3_000_001])
+def test_stream_probe_two_outputs(n_packs):
+    from teletron_amd import cabi
+    g = torch.Generator().manual_seed(n_packs)
+    a = torch.randint(-2**31, 2**31 - 1, (n_packs * 4 + 4,), generator=g, dtype=torch.int32).to(DEV)
+    out0, out1 = torch.full_like(a, 7), torch.full_like(a, 9)
+    stream = torch.cuda.current_stream().cuda_stream
+    cabi.call("tt_stream_probe_two_outputs", out0.data_ptr(), out1.data_ptr(), a.data_ptr(), n_packs * 16, stream)
+    assert torch.equal(out0[:n_packs * 4], a[:n_packs * 4])
+    assert torch.equal(out1[:n_packs * 4], ~a[:n_packs * 4])
+    assert torch.all(out0[n_packs * 4:] == 7) and torch.all(out1[n_packs * 4:] == 9)
+    lib = cabi.load()
+    assert lib.tt_stream_probe_two_outputs(out0.data_ptr(), None, a.data_ptr(), 64, None) == cabi.TT_ERR_INVALID_ARGUMENT
+    assert lib.tt_stream_probe_two_outputs(out0.data_ptr(), out1.data_ptr(), a.data_ptr(), 24, None) == cabi.TT_ERR_UNSUPPORTED
+
+
 def test_stream_probe_errors():
     from teletron_amd import cabi
     lib = cabi.load()
