@@ -99,13 +99,19 @@ TT_API size_t tt_adaln_backward_workspace_bytes(int64_t rows, int64_t cols, int6
 /* tt_adaln_backward for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without the
  * workspace, same kernels, same results bit for bit.  No counterpart in the reference.  The
- * partial column sums live in a device array inside the library, TT_STATIC_WORKSPACE_BYTES
- * (16 MiB) per GPU, held from the first call on that GPU until the process ends; the call
- * performs no hipMalloc / hipFree.  A shape whose launch plan needs more (what
- * tt_adaln_backward_workspace_bytes() returns; 10.2 MB at rows 75600, cols 5120) is refused
- * with TT_ERR_STATIC_LIMIT.  All calls on one GPU share the array: two calls that overlap in
- * time on the same GPU (different streams or host threads) race and give wrong dscale / dshift;
- * calls that follow each other on one stream are safe (nothing in the array has to start at zero).
+ * scratch memory (partial column sums) is a device array inside the library,
+ * TT_STATIC_WORKSPACE_BYTES (16 MiB); every GPU on which the library's code is loaded holds its
+ * own copy until the process ends, whether or not this entry point is ever called.  The call
+ * performs no hipMalloc / hipFree.  The first call on a GPU looks up that GPU's address of the
+ * array (hipGetSymbolAddress) and the launch plan's device properties; a call with rows == 0 does
+ * only that and touches no pointer, for callers that want this set-up done at a chosen moment.
+ * A shape that needs more scratch than the array holds is refused with TT_ERR_STATIC_LIMIT: the
+ * need is what tt_adaln_backward_workspace_bytes() returns (10.2 MB at rows 75600, cols 5120), or
+ * rows * 8 bytes when cols is not a multiple of 8 or a tensor is not 16-byte aligned.  All calls
+ * on one GPU share the array: two calls that overlap in time on the same GPU (different streams
+ * or host threads, or two replays of graphs that captured it) race and give wrong dscale /
+ * dshift; calls that follow each other on one stream are safe (nothing in the array has to
+ * start at zero).
  */
 #define TT_STATIC_WORKSPACE_BYTES (16u << 20)
 TT_API int tt_adaln_backward_static(void* dx, float* dscale, float* dshift,

@@ -438,7 +438,7 @@ const char* tt_error_string(int code) {
     case TT_ERR_UNSUPPORTED: return "unsupported shape or alignment";
     case TT_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case TT_ERR_HIP: return "HIP runtime error (see tt_last_hip_error)";
-    case TT_ERR_STATIC_LIMIT: return "shape needs more than TT_STATIC_WORKSPACE_BYTES of scratch: use the entry point that takes a workspace";
+    case TT_ERR_STATIC_LIMIT: return "shape needs more than TT_STATIC_WORKSPACE_BYTES of scratch (partial sums, or rows * 8 bytes on the element-wise path): use the entry point that takes a workspace";
     default: return "unknown error code";
   }
 }
@@ -506,10 +506,10 @@ int tt_adaln_backward(void* dx, float* dscale, float* dshift, const void* dy, co
 int tt_adaln_backward_static(void* dx, float* dscale, float* dshift, const void* dy, const void* x,
                              const void* scale, int64_t rows, int64_t cols, int64_t rows_per_batch, float eps,
                              void* stream) {
-  if (rows == 0) return TT_OK;
   void* ws = nullptr;
-  int rc = static_scratch(&ws);
+  int rc = static_scratch(&ws);   // per-device set-up on the first call; a rows == 0 call does only this
   if (rc != TT_OK) return rc;
+  if (rows == 0) return TT_OK;
   rc = tt_adaln_backward(dx, dscale, dshift, dy, x, scale, ws, TT_STATIC_WORKSPACE_BYTES,
                          rows, cols, rows_per_batch, eps, stream);
   return rc == TT_ERR_WORKSPACE ? TT_ERR_STATIC_LIMIT : rc;

@@ -4,6 +4,11 @@
 #include <torch/extension.h>
 #include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "teletron_op.h"
 
@@ -32,8 +37,25 @@ inline void check_shape(int64_t rows, int64_t cols) {
 inline void* current_stream(const torch::Tensor& t) {
   return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
 }
+// Backward workspace (per-workgroup partial sums): one tensor per (device, stream), grown on demand
+// and reused from call to call, so a backward call does not go to the allocator (the reference
+// allocates its fp32 [32, C] scratch on every call, teletron_op/fused_rmsnorm/weight_backward.cu:229).
+// Launches on one stream run in order, so consecutive calls never overlap in it.  A stream under
+// graph capture gets memory of its own from the capture's pool: the graph keeps the pointer.
+// The cache is never destroyed (the HIP runtime may be gone by the time static destructors run).
 inline torch::Tensor workspace(size_t bytes, const torch::Tensor& ref) {
-  return at::empty({static_cast<int64_t>(bytes)}, at::TensorOptions().dtype(at::kByte).device(ref.device()));
+  const auto opts = at::TensorOptions().dtype(at::kByte).device(ref.device());
+  const int64_t need = static_cast<int64_t>(bytes < 16 ? 16 : bytes);
+  hipStream_t stream = c10::hip::getCurrentHIPStream(ref.device().index()).stream();
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+  if (capturing != hipStreamCaptureStatusNone) return at::empty({need}, opts);
+  static std::mutex mu;
+  static auto* cache = new std::map<std::pair<int, hipStream_t>, torch::Tensor>();
+  std::lock_guard<std::mutex> lock(mu);
+  torch::Tensor& ws = (*cache)[{static_cast<int>(ref.device().index()), stream}];
+  if (!ws.defined() || ws.numel() < need) ws = at::empty({need}, opts);
+  return ws;
 }
 inline void check_status(int rc, const char* what) {
   TORCH_CHECK(rc == TT_OK, what, " failed: ", tt_error_string(rc),

@@ -27,9 +27,20 @@ from torch.autograd import Function
 from . import ops
 
 
+def _check_row_groups(x, *params):
+    """The ops read a parameter as one vector per consecutive group of rows of the flattened input.
+    A parameter with the input's rank is shaped for broadcasting, and must then mean the same thing
+    ([B, 1, C] for x [B, S, C] does; [1, S, C] with B > 1 does not): refused rather than misread."""
+    for p in params:
+        if p is not None and x.dim() >= 3 and p.dim() == x.dim() and ops.row_groups(x, p) is None:
+            raise ValueError(f"a parameter of shape {tuple(p.shape)} does not broadcast over consecutive groups of rows "
+                             f"of an input of shape {tuple(x.shape)}")
+
+
 def _adaln_forward(ctx, x, scale, shift, epsilon, cols):
     if x.numel() % cols != 0 or x.shape[-1] != cols:
         raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols}")
+    _check_row_groups(x, scale, shift)
     ctx.eps = float(epsilon)
     ctx.scale_meta = (scale.shape, scale.dtype)
     ctx.shift_meta = (shift.shape, shift.dtype)
@@ -175,6 +186,7 @@ def rope_table_from_cos_sin(cos: torch.Tensor, sin: torch.Tensor, extra_tokens: 
 
 
 def _gate_forward(ctx, x, gate, residual):
+    _check_row_groups(x, gate)
     ctx.gate_meta = (gate.shape, gate.dtype)
     gate_c = gate.detach().to(torch.bfloat16).contiguous()
     residual = residual.contiguous()
@@ -238,6 +250,7 @@ class ResidualNormFunction(Function):
     @staticmethod
     def forward(ctx, x, residual, gate, scale, shift, epsilon, affine, grad_reduce=None):
         ctx.eps, ctx.affine, ctx.grad_reduce = float(epsilon), bool(affine), grad_reduce
+        _check_row_groups(x, gate, scale, shift)
         ctx.set_materialize_grads(False)
         ctx.metas = [None if t is None else (t.shape, t.dtype) for t in (gate, scale, shift)]
         bf = torch.bfloat16

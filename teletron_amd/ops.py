@@ -10,6 +10,7 @@ consecutive groups, group ``b`` using modulation vector ``b``.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import Optional, Tuple
 
 import torch
@@ -66,6 +67,29 @@ def _inverse(perm):
     return inv
 
 
+def row_groups(x: torch.Tensor, p) -> Optional[int]:
+    """The fused kernels modulate consecutive groups of rows of the flattened ``x`` with one vector
+    each.  Returns the number of groups if broadcasting ``p`` against ``x`` means exactly that
+    (``p`` equals ``x`` in some leading dimensions, is 1 in every later one and ``C`` in the last:
+    ``[C]``, ``[1, 1, C]``, ``[B, 1, C]``, ``[B, S, C]`` for ``x [B, S, C]``), else None
+    (``[1, S, C]`` with ``B > 1``, a wider last dimension, more dimensions than ``x`` ...)."""
+    n = x.dim()
+    if not isinstance(p, torch.Tensor) or p.dim() < 1 or p.dim() > n or n < 1:
+        return None
+    shape = (1,) * (n - p.dim()) + tuple(p.shape)
+    if shape[-1] != x.shape[-1]:
+        return None
+    groups, broadcasting = 1, False
+    for i in range(n - 1):
+        if shape[i] == x.shape[i] and (not broadcasting or shape[i] == 1):
+            groups *= shape[i]
+        elif shape[i] == 1:
+            broadcasting = True
+        else:
+            return None
+    return groups
+
+
 def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int, int]:
     rows = x.numel() // cols
     nb = scale.numel() // cols
@@ -75,6 +99,17 @@ def _batches(x: torch.Tensor, scale: torch.Tensor, cols: int) -> Tuple[int, int,
 
 
 _WORKSPACES = {}   # (device index, stream handle) -> uint8 tensor, grown on demand
+_WORKSPACES_LOCK = threading.Lock()   # backward runs on autograd's threads, one per device
+# the element-wise path's row statistics (rows * 8 bytes) are only kept between calls up to this size
+_WORKSPACE_KEEP_BYTES = 64 << 20
+
+
+def clear_workspaces() -> None:
+    """Drop the cached backward workspaces (one per device and stream that ever ran a backward, about
+    10 MB each at the Wan-14B shape).  Safe between steps; kernels already launched keep their memory
+    until they finish (the caching allocator frees in stream order)."""
+    with _WORKSPACES_LOCK:
+        _WORKSPACES.clear()
 
 
 def _workspace(lib_bytes: int, rows: int, *tensors: torch.Tensor) -> torch.Tensor:
@@ -92,10 +127,12 @@ def _workspace(lib_bytes: int, rows: int, *tensors: torch.Tensor) -> torch.Tenso
         # capture's private pool), never the shared buffer
         return torch.empty(need, dtype=torch.uint8, device=dev)
     key = (dev.index, _stream(tensors[0]))
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < need:
-        ws = torch.empty(need, dtype=torch.uint8, device=dev)
-        _WORKSPACES[key] = ws
+    with _WORKSPACES_LOCK:
+        ws = _WORKSPACES.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(need, dtype=torch.uint8, device=dev)
+            if need <= _WORKSPACE_KEEP_BYTES:
+                _WORKSPACES[key] = ws
     return ws
 
 

@@ -111,7 +111,7 @@ class DeferredNorm:
         # (1 + scale) was rounded to the activation dtype by the caller.  Subtracting 1 again is
         # exact while 0.5 <= 1 + scale <= 2 (Sterbenz); outside that range it can lose the last
         # bit of the rounded factor, far below the bf16 resolution of the output.
-        if not _same_dtype(self.x, shift, self.one_plus_scale):   # wider modulation: eager, which promotes
+        if not modulation_fusable(self.x, shift, self.one_plus_scale):   # eager: promotes / broadcasts as written
             return self.materialize() * self.one_plus_scale + shift
         return modulate_token(self, shift, self.one_plus_scale - 1)
 
@@ -127,12 +127,44 @@ class DeferredNorm:
             "`modulate(...)` or used as `norm(x) * (1 + scale) + shift`; call .materialize() for anything else")
 
 
+MAX_COLS = 32768            # widest row the kernels take
+MAX_ROW_GROUPS = 65535      # the kernels take one modulation vector per grid row
+MIN_ROWS_PER_GROUP = 8      # below this the eager expression is the faster one
+
+
+row_groups = ops.row_groups
+
+
+def modulation_fusable(x: torch.Tensor, *params) -> bool:
+    """True where the fused kernels compute what the eager expression computes: every parameter on
+    ``x``'s device and of its dtype (eager promotes to a wider one), broadcasting per row group (see
+    :func:`row_groups`), all with the same number of groups, at most ``MAX_ROW_GROUPS`` of them and
+    at least ``MIN_ROWS_PER_GROUP`` rows in each.  Everything else stays on the original path."""
+    if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16 and x.dim() >= 1 and x.numel() > 0
+            and x.shape[-1] <= MAX_COLS):
+        return False
+    groups = None
+    for p in params:
+        if p is None:
+            continue
+        g = row_groups(x, p)
+        if g is None or p.dtype != x.dtype or p.device != x.device or (groups is not None and g != groups):
+            return False
+        groups = g
+    if groups is None:
+        return True
+    rows = x.numel() // x.shape[-1]
+    return groups == 1 or (groups <= MAX_ROW_GROUPS and rows // groups >= MIN_ROWS_PER_GROUP)
+
+
 def modulate_token(token: DeferredNorm, shift: torch.Tensor, scale: torch.Tensor,
                    grad_reduce: Optional[Callable] = None) -> torch.Tensor:
     x = token.x
-    if not _same_dtype(x, shift, scale):      # wider modulation: the eager expression, which promotes
+    if not modulation_fusable(x, shift, scale):
+        # wider modulation (eager promotes), per-token or otherwise unsupported shapes: the eager expression
         if grad_reduce is not None:
-            raise TypeError("the gradient-reducing fused modulation needs shift / scale in the activation's dtype")
+            raise TypeError("the gradient-reducing fused modulation needs shift / scale in the activation's dtype, "
+                            "one vector per consecutive group of rows")
         return token.materialize() * (1 + scale) + shift
     if grad_reduce is not None:
         return AdaLNGradReduceFunction.apply(x, scale, shift, token.eps, x.shape[-1], grad_reduce)
@@ -171,7 +203,13 @@ def fused_gate(original: Callable, grad_reduce: Optional[Callable] = None) -> Ca
 def _is_cp_callable(attr: str, fn) -> bool:
     """A context-parallel gradient-reducing callable, under its own name or assigned to another
     attribute (``norm1.modulate = self.modulate_with_cp_grad_reduce``, hunyuan/parallel_model.py:239-244)."""
-    return attr in CP_ATTRS or getattr(fn, "__name__", "") in CP_ATTRS
+    while True:
+        if attr in CP_ATTRS or getattr(fn, "__name__", "") in CP_ATTRS:
+            return True
+        inner = getattr(fn, "__wrapped__", None)      # a callable this module has wrapped already
+        if inner is None:
+            return False
+        fn = inner
 
 
 def _several_ranks() -> bool:
@@ -183,9 +221,11 @@ class DeferredLayerNorm(nn.Module):
     """Stands in for ``nn.LayerNorm(dim, eps, elementwise_affine=False)``; parameter-free, so
     replacing the original changes no state-dict key."""
 
-    def __init__(self, dim: int, eps: float):
+    def __init__(self, dim: int, eps: float, original: Optional[nn.Module] = None):
         super().__init__()
         self.normalized_shape, self.eps = (dim,), eps
+        # the module this one stands in for, kept for swap_out; not registered as a child
+        self.__dict__["_tt_original"] = original
 
     def forward(self, x: torch.Tensor):
         if x.is_cuda and x.dtype == torch.bfloat16:
@@ -211,14 +251,16 @@ def _same_dtype(x: torch.Tensor, *params) -> bool:
 
 
 def _fused_rmsnorm_forward(self, x: torch.Tensor) -> torch.Tensor:
-    if x.is_cuda and x.dtype == torch.bfloat16 and _same_dtype(x, self.weight):
+    if (x.is_cuda and x.dtype == torch.bfloat16 and _same_dtype(x, self.weight) and x.dim() >= 1 and x.numel() > 0
+            and self.weight.shape[0] == x.shape[-1] <= MAX_COLS and self.weight.device == x.device):
         return RMSNormModelFunction.apply(x, self.weight, self.eps, x.shape[-1])
     return type(self).forward(self, x)
 
 
 def _gate_fusable(x, gate, residual) -> bool:
-    return (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16 and isinstance(residual, torch.Tensor)
-            and residual.dtype == torch.bfloat16 and x.shape == residual.shape and _same_dtype(x, gate))
+    return (isinstance(x, torch.Tensor) and isinstance(residual, torch.Tensor) and residual.dtype == torch.bfloat16
+            and x.shape == residual.shape and residual.device == x.device and x.shape[-1] % 8 == 0
+            and modulation_fusable(x, gate))
 
 
 def _fused_gate_forward(self, x, gate, residual):
@@ -251,10 +293,14 @@ def fused_dit_block_forward(self, x, context, t_mod, freqs):
     """``DiTBlock.forward`` (``wan_model.py:231-244``; ``parallel_wan_model.py:18-37`` is the same
     sequence) with the norm + modulate pairs and both residual updates on the fused kernels.  The
     sub-modules (``self_attn``, ``cross_attn``, ``ffn``) and all parameters are used as they are."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and _same_dtype(x, t_mod, self.norm3.weight, self.norm3.bias)):
+    if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.bfloat16 and isinstance(t_mod, torch.Tensor)
+            and _same_dtype(x, t_mod, self.norm3.weight, self.norm3.bias) and x.dim() == 3 and t_mod.dim() == 3
+            and t_mod.shape[1] == 6 and ops.residual_norm_supported(x)):
         return type(self).forward(self, x, context, t_mod, freqs)
     shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = (
         self.modulation.to(dtype=t_mod.dtype, device=t_mod.device) + t_mod).chunk(6, dim=1)
+    if not modulation_fusable(x, shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp):
+        return type(self).forward(self, x, context, t_mod, freqs)
     # context-parallel block told how to reduce: the gradients of the six modulation chunks pass through it
     reduce = self.__dict__.get("_tt_grad_reduce")
     input_x = adaln_modulate(x, shift_msa, scale_msa, self.norm1.eps, reduce)
@@ -430,8 +476,10 @@ def fused_hunyuan_block_forward(self, hidden_states, encoder_hidden_states, temb
     attn_output, context_attn_output = self.attn(hidden_states=norm_hidden_states,
                                                  encoder_hidden_states=norm_encoder_hidden_states,
                                                  attention_mask=attention_mask, image_rotary_emb=freqs_cis)
-    if (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and attn_output.dtype == torch.bfloat16
-            and _same_dtype(hidden_states, gate_msa, shift_mlp, scale_mlp)):
+    if (isinstance(attn_output, torch.Tensor) and attn_output.dtype == torch.bfloat16
+            and attn_output.shape == hidden_states.shape and ops.residual_norm_supported(hidden_states)
+            and all(isinstance(t, torch.Tensor) and t.dim() == 2 for t in (gate_msa, shift_mlp, scale_mlp))
+            and modulation_fusable(hidden_states, gate_msa.unsqueeze(1), shift_mlp[:, None], scale_mlp[:, None])):
         hidden_states, norm_hidden_states = residual_adaln(hidden_states, attn_output, gate_msa.unsqueeze(1),
                                                            shift_mlp[:, None], scale_mlp[:, None], self.norm2.eps)
     else:
@@ -573,8 +621,59 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
                 ln = getattr(module, attr, None)
                 dim = _plain_layernorm_dim(ln)
                 if dim is not None:
-                    setattr(module, attr, DeferredLayerNorm(dim, ln.eps))
+                    setattr(module, attr, DeferredLayerNorm(dim, ln.eps, ln))
                     counts["layernorm"] += 1
+    return counts
+
+
+_FUSED_FORWARDS = (_fused_rmsnorm_forward, _fused_gate_forward, fused_dit_block_forward, fused_hunyuan_block_forward,
+                   fused_hunyuan_single_block_forward, fused_self_attention_forward)
+
+
+def _unwrap_attr(obj, attr: str) -> bool:
+    """Put back what ``fused_modulate`` / ``fused_gate`` wrapped under ``obj.attr``."""
+    fn = obj.__dict__.get(attr) if isinstance(obj, nn.Module) else getattr(obj, attr, None)
+    original = getattr(fn, "__wrapped__", None)
+    if fn is None or original is None:
+        return False
+    method = getattr(type(obj), attr, None) if isinstance(obj, nn.Module) else None
+    if method is not None and getattr(original, "__self__", None) is obj and getattr(original, "__func__", None) is method:
+        del obj.__dict__[attr]            # the wrapper shadowed the class's own method: uncover it
+    else:
+        setattr(obj, attr, original)
+    return True
+
+
+def swap_out(model: nn.Module, namespaces: Iterable[object] = ()) -> dict:
+    """Undo every patch :func:`swap_in` made on ``model`` and ``namespaces``: instance ``forward``s are
+    removed (the class's own method shows again), wrapped ``modulate`` / ``gate`` callables and
+    attention processors are put back, and each :class:`DeferredLayerNorm` gives way to the very
+    module it replaced.  Parameters were never touched, so state-dict keys are the same before
+    ``swap_in``, between the two calls and after.  Returns counts in ``swap_in``'s categories."""
+    counts = {"rmsnorm": 0, "layernorm": 0, "modulate": 0, "gate": 0, "block": 0, "attention": 0, "processor": 0}
+    kind = {_fused_rmsnorm_forward: "rmsnorm", _fused_gate_forward: "gate", fused_self_attention_forward: "attention"}
+    for ns in namespaces:
+        if _unwrap_attr(ns, "modulate"):
+            counts["modulate"] += 1
+    for module in list(model.modules()):
+        fwd = module.__dict__.get("forward")
+        if isinstance(fwd, types.MethodType) and fwd.__func__ in _FUSED_FORWARDS:
+            del module.__dict__["forward"]
+            counts[kind.get(fwd.__func__, "block")] += 1
+        module.__dict__.pop("_tt_grad_reduce", None)
+        if isinstance(getattr(module, "processor", None), FusedHunyuanAttnProcessor):
+            module.processor = module.processor.original
+            counts["processor"] += 1
+        for attr in MODULATE_ATTRS:
+            if _unwrap_attr(module, attr):
+                counts["modulate"] += 1
+        for attr in GATE_ATTRS + ("gate",):
+            if not isinstance(module.__dict__.get("_modules", {}).get(attr), nn.Module) and _unwrap_attr(module, attr):
+                counts["gate"] += 1
+        for name, child in list(module.named_children()):
+            if isinstance(child, DeferredLayerNorm) and child.__dict__.get("_tt_original") is not None:
+                setattr(module, name, child.__dict__["_tt_original"])
+                counts["layernorm"] += 1
     return counts
 
 

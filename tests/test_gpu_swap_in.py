@@ -462,3 +462,95 @@ def test_context_parallel_wan_block_forward_with_a_reduce_hook(monkeypatch):
     worst = max((e, n) for n, e in errs.items() if not n.endswith("cross_attn.k.bias"))
     assert worst[0] < 2e-2, worst
     assert max(e for n, e in errs.items() if n.endswith("cross_attn.k.bias")) < 4e-2
+
+
+class ModulatedNorm(nn.Module):
+    """norm + modulation written both ways the models write it: modulate(norm(x), shift, scale)
+    through the namespace's function (wan_model.py:236) and inline (wan_model.py:277)."""
+
+    def __init__(self, dim, inline):
+        super().__init__()
+        self.norm = nn.LayerNorm(dim, eps=1e-6, elementwise_affine=False)
+        self.gate, self.inline = GateModule(), inline
+
+    def forward(self, x, shift, scale, gate):
+        h = self.norm(x) * (1 + scale) + shift if self.inline else ns.modulate(self.norm(x), shift, scale)
+        return self.gate(x, gate, h)
+
+
+ModulatedNorm.__name__ = "Head"          # an owner class swap_in knows (its `norm` is replaced)
+
+REFUSED = {
+    # name: (shift shape, scale shape, gate shape) for x [2, 96, 256]
+    "per_token_modulation": ((2, 96, 256), (2, 96, 256), (2, 1, 256)),
+    "per_token_shared_by_samples": ((1, 96, 256), (1, 96, 256), (1, 1, 256)),
+    "scale_and_shift_of_different_shapes": ((1, 1, 256), (2, 1, 256), (2, 1, 256)),
+    "per_token_gate": ((2, 1, 256), (2, 1, 256), (2, 96, 256)),
+    "gate_shared_by_samples_per_token": ((2, 1, 256), (2, 1, 256), (1, 96, 256)),
+}
+
+
+@pytest.mark.parametrize("inline", [False, True])
+@pytest.mark.parametrize("case", sorted(REFUSED))
+def test_shapes_the_kernels_refuse_take_the_original_path(case, inline):
+    """Modulation shapes the fused kernels do not cover (per-token vectors, scale and shift that
+    broadcast differently) ran in the eager model; after swap_in they must still run, and give the
+    eager result (the part that cannot be fused is the original expression, bit for bit)."""
+    from teletron_amd import swap_in as S
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s, scale=1.0: (scale * torch.randn(*s, generator=g)).to(torch.bfloat16).to(DEV)
+    sh_shape, sc_shape, g_shape = REFUSED[case]
+    x, dy = mk(2, 96, 256), mk(2, 96, 256)
+    inputs = [x, mk(*sh_shape, scale=0.2), mk(*sc_shape, scale=0.2), mk(*g_shape, scale=0.5)]
+    model = ModulatedNorm(256, inline).to(DEV)
+    out_e, gin_e, _ = run(model, inputs, dy)
+    counts = S.swap_in(model, [ns])
+    try:
+        assert counts["layernorm"] == 1 and counts["gate"] == 1
+        out_f, gin_f, _ = run(model, inputs, dy)          # must not raise
+    finally:
+        S.swap_out(model, [ns])
+    assert ns.modulate is modulate
+    fused_gate = "gate" not in case                        # the gate is fused where its own shape allows it
+    fused_norm = "gate" in case
+    if not fused_gate and not fused_norm:
+        assert torch.equal(out_f, out_e)
+        for a, b in zip(gin_f, gin_e):
+            assert torch.equal(a, b)
+    else:
+        assert rel(out_f, out_e) < 5e-3
+        for a, b in zip(gin_f, gin_e):
+            assert rel(a, b) < 2e-2
+
+
+def test_function_refuses_a_parameter_that_is_not_per_row_group():
+    """Called directly, the autograd Functions read a parameter as one vector per consecutive group
+    of rows; a [1, S, C] tensor against x [B, S, C] means something else under broadcasting and is
+    refused instead of being misread."""
+    from teletron_amd import AdaLNModelFunction, GateResidualFunction
+    x = torch.randn(2, 32, 64, device=DEV).to(torch.bfloat16)
+    per_token = torch.zeros(1, 32, 64, device=DEV, dtype=torch.bfloat16)
+    per_sample = torch.zeros(2, 1, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="consecutive groups of rows"):
+        AdaLNModelFunction.apply(x, per_token, per_token, 1e-6, 64)
+    with pytest.raises(ValueError, match="consecutive groups of rows"):
+        GateResidualFunction.apply(x, per_token, x)
+    AdaLNModelFunction.apply(x, per_sample, per_sample, 1e-6, 64)
+    AdaLNModelFunction.apply(x, torch.zeros(2, 32, 64, device=DEV, dtype=torch.bfloat16), per_sample.expand(2, 32, 64), 1e-6, 64)
+
+
+def test_swap_out_on_the_gpu_model_gives_back_the_eager_results():
+    from teletron_amd import swap_in as S
+    torch.manual_seed(0)
+    dim, bsz, seq = 256, 2, 96
+    model = Model(dim).to(DEV).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(1)
+    mk = lambda *s, scale=1.0: (scale * torch.randn(*s, generator=g)).to(torch.bfloat16).to(DEV)
+    inputs = [mk(bsz, seq, dim), mk(bsz, 6, dim, scale=0.2), mk(bsz, 2, dim, scale=0.2), mk(bsz, dim)]
+    dy = mk(bsz, seq, 64)
+    out_e, gin_e, gp_e = run(model, inputs, dy)
+    counts = S.swap_in(model, [ns])
+    assert S.swap_out(model, [ns]) == counts and ns.modulate is modulate
+    out_r, gin_r, gp_r = run(model, inputs, dy)
+    assert torch.equal(out_r, out_e) and all(torch.equal(a, b) for a, b in zip(gin_r, gin_e))
+    assert all(torch.equal(gp_r[n], gp_e[n]) for n in gp_e)
