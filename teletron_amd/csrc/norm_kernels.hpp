@@ -1084,22 +1084,19 @@ __global__ __launch_bounds__(1024) void reduce_partials(void* __restrict__ out0,
   for (int acc = 0; acc < NACC; ++acc) s[acc] = 0.f;
   if (c < cols) {
     const float* base = partials + (size_t)b * n_partials * NACC * cols + c;
-    // 8 independent loads per accumulator in flight; the sum order stays fixed.
-    int j = wave;
-    for (; j + 7 * 16 < n_partials; j += 8 * 16) {
+    // 8 independent loads per accumulator in flight, in the ragged last round too (a missing
+    // partial contributes +0.0f, which changes no sum); the sum order stays fixed.
+    for (int j = wave; j < n_partials; j += 8 * 16) {
       float t[8][NACC];
 #pragma unroll
       for (int u = 0; u < 8; ++u)
 #pragma unroll
-        for (int acc = 0; acc < NACC; ++acc) t[u][acc] = base[((size_t)(j + u * 16) * NACC + acc) * cols];
+        for (int acc = 0; acc < NACC; ++acc)
+          t[u][acc] = j + u * 16 < n_partials ? base[((size_t)(j + u * 16) * NACC + acc) * cols] : 0.f;
 #pragma unroll
       for (int u = 0; u < 8; ++u)
 #pragma unroll
         for (int acc = 0; acc < NACC; ++acc) s[acc] += t[u][acc];
-    }
-    for (; j < n_partials; j += 16) {
-#pragma unroll
-      for (int acc = 0; acc < NACC; ++acc) s[acc] += base[((size_t)j * NACC + acc) * cols];
     }
   }
 #pragma unroll
