@@ -82,6 +82,18 @@ def torch_ext_path(name: str) -> Path:
     return PKG_DIR / (name + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
+def is_current() -> bool:
+    """True when the library and the glue modules exist and each is newer than every source it is built from."""
+    glue = [torch_ext_path(n) for n in TORCH_EXT_MODULES]
+    if not LIB_PATH.exists() or not all(g.exists() for g in glue):
+        return False
+    header = REPO_ROOT / "include" / "teletron_op.h"
+    newest = lambda files: max(f.stat().st_mtime for f in files)
+    lib_srcs = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.hpp")) + [header]
+    glue_srcs = list((CSRC / "torch_ext").glob("*")) + [header]
+    return LIB_PATH.stat().st_mtime > newest(lib_srcs) and min(g.stat().st_mtime for g in glue) > newest(glue_srcs)
+
+
 def build_torch_extensions(force: bool = True, verbose: bool = True):
     """Compile the pybind / TORCH_LIBRARY glue modules (host C++ only, g++) against the
     installed torch and link them to libteletron_op.so.  They hold no kernels."""

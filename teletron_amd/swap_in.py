@@ -56,6 +56,7 @@ forward is not installed on context-parallel blocks then).
 from __future__ import annotations
 
 import os
+import threading
 import types
 import weakref
 from typing import Callable, Iterable, Optional
@@ -342,36 +343,51 @@ def fused_self_attention_forward(self, x, freqs):
 class _RotaryTableCache:
     """The fp32 (cos, sin) table of ``rope_table_from_cos_sin`` for the rotary pair a model hands to
     all of its blocks in one forward pass: built on first use, reused while the very same tensor
-    objects (held weakly) are passed again unmodified, dropped when they are freed.  One entry per
-    number of appended text tokens."""
+    objects (held weakly) are passed again unmodified, dropped when they are freed, and dropped at
+    the start of every forward pass of the model ``swap_in`` was called on (a pre-forward hook), so
+    that values changed in place between two passes are never missed; that matters for tensors made
+    under ``torch.inference_mode()``, which keep no version counter to see such a change by.  One
+    entry per number of appended text tokens."""
 
     def __init__(self):
         self.entries = {}
+        self.lock = threading.RLock()   # re-entrant: a weak-reference callback may fire while it is held
 
     @staticmethod
     def _versions(cos, sin):
         try:
             return cos._version, sin._version
-        except RuntimeError:        # tensors made under torch.inference_mode() keep no version counter:
-            return None             # the same objects are then taken to hold the same values
+        except RuntimeError:        # inference-mode tensors keep no version counter: within one forward
+            return None             # pass the same objects are taken to hold the same values
+
+    def clear(self):
+        with self.lock:
+            self.entries.clear()
 
     def get(self, cos: torch.Tensor, sin: torch.Tensor, extra_tokens: int) -> torch.Tensor:
-        e = self.entries.get(extra_tokens)
         versions = self._versions(cos, sin)
-        if e is not None and e[0]() is cos and e[1]() is sin and e[2] == versions:
-            return e[3]
+        with self.lock:
+            e = self.entries.get(extra_tokens)
+            if e is not None and e[0]() is cos and e[1]() is sin and e[2] == versions:
+                return e[3]
         table = rope_table_from_cos_sin(cos, sin, extra_tokens=extra_tokens)
 
         def drop(ref, key=extra_tokens):          # the pair is gone: so is the table built from it
-            held = self.entries.get(key)
-            if held is not None and ref in (held[0], held[1]):
-                del self.entries[key]
+            with self.lock:
+                held = self.entries.get(key)
+                if held is not None and ref in (held[0], held[1]):
+                    del self.entries[key]
 
-        self.entries[extra_tokens] = (weakref.ref(cos, drop), weakref.ref(sin, drop), versions, table)
+        with self.lock:
+            self.entries[extra_tokens] = (weakref.ref(cos, drop), weakref.ref(sin, drop), versions, table)
         return table
 
 
 _ROTARY_TABLES = _RotaryTableCache()
+
+
+def _drop_rotary_tables(module, args):
+    _ROTARY_TABLES.clear()
 
 
 def split_tokens(t: torch.Tensor, n_text: int):
@@ -623,6 +639,9 @@ def swap_in(model: nn.Module, namespaces: Iterable[object] = (), rmsnorm: bool =
                 if dim is not None:
                     setattr(module, attr, DeferredLayerNorm(dim, ln.eps, ln))
                     counts["layernorm"] += 1
+    if counts["processor"] and "_tt_rotary_hook" not in model.__dict__:
+        # the processors share one rotary table per forward pass of `model`: rebuilt at the start of each
+        model.__dict__["_tt_rotary_hook"] = model.register_forward_pre_hook(_drop_rotary_tables)
     return counts
 
 
@@ -655,6 +674,10 @@ def swap_out(model: nn.Module, namespaces: Iterable[object] = ()) -> dict:
     for ns in namespaces:
         if _unwrap_attr(ns, "modulate"):
             counts["modulate"] += 1
+    hook = model.__dict__.pop("_tt_rotary_hook", None)
+    if hook is not None:
+        hook.remove()
+        _ROTARY_TABLES.clear()
     for module in list(model.modules()):
         fwd = module.__dict__.get("forward")
         if isinstance(fwd, types.MethodType) and fwd.__func__ in _FUSED_FORWARDS:

@@ -206,3 +206,37 @@ def test_glue_modules_find_the_library_by_name_not_by_build_path():
         assert "libteletron_op.so" in needed, needed
         assert not [n for n in needed if "/" in n], needed
         assert "$ORIGIN" in out
+
+
+def test_installed_form_exports_the_reference_module_names(tmp_path):
+    """What teletron_op/install.sh leaves behind (teletron_op/install.sh:1-9): `import fused_adaln` and
+    `import fused_rmsnorm` work from anywhere.  setup.py is run on a copy of the tree (the built
+    libraries travel with it and are reused), installing into a scratch directory; a fresh interpreter
+    started elsewhere must then find both modules, with the reference's function names, and the C ABI."""
+    import shutil
+    import subprocess
+    import sys
+    from pathlib import Path
+    repo = Path(REPO)
+    src = tmp_path / "src"
+    src.mkdir()
+    shutil.copy2(repo / "setup.py", src / "setup.py")
+    shutil.copytree(repo / "include", src / "include")
+    shutil.copytree(repo / "teletron_amd", src / "teletron_amd",
+                    ignore=shutil.ignore_patterns("__pycache__", "build"))
+    site = tmp_path / "site"
+    r = subprocess.run([sys.executable, "-m", "pip", "install", "--no-build-isolation", "--no-index", "--no-deps",
+                        "--quiet", "--target", str(site), str(src)], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout + r.stderr
+    code = ("import fused_adaln, fused_rmsnorm, teletron_amd, torch\n"
+            "assert callable(fused_adaln.torch_launch_adaln_forward) and callable(fused_adaln.torch_launch_adaln_backward)\n"
+            "assert callable(fused_rmsnorm.torch_launch_rms_forward) and callable(fused_rmsnorm.torch_launch_rms_backward)\n"
+            "assert hasattr(torch.ops.layernorm_block_smem, 'torch_launch_adaln_forward')\n"
+            "assert hasattr(torch.ops.Fused_RMSNorm, 'torch_launch_rms_backward')\n"
+            "assert teletron_amd.cabi.load().tt_version() >= 100\n"
+            "print(fused_adaln.__file__)\n")
+    env = {k: v for k, v in __import__("os").environ.items() if k != "PYTHONPATH"}
+    env["PYTHONPATH"] = str(site)
+    r = subprocess.run([sys.executable, "-c", code], cwd=str(tmp_path), env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert str(site) in r.stdout

@@ -122,3 +122,24 @@ def test_modulation_fusable_refuses_cpu_and_wide_dtypes():
     p = torch.empty(2, 1, 16, dtype=torch.bfloat16)
     assert not S.modulation_fusable(x, p)                                 # CPU tensors never take the kernels
     assert not S.modulation_fusable(x.float(), p.float())
+
+
+def test_rotary_tables_are_rebuilt_at_every_forward_pass_of_the_swapped_model():
+    """Tensors made under torch.inference_mode() keep no version counter, so an in-place change of the
+    rotary pair between two passes cannot be seen on the tensors themselves: the table cache is
+    emptied by a pre-forward hook on the model swap_in was called on, and swap_out removes the hook."""
+    model = H.TwoStreamModel(heads=2, head_dim=64)
+    S.swap_in(model, blocks=True)
+    assert "_tt_rotary_hook" in model.__dict__ and len(model._forward_pre_hooks) == 1
+    with torch.inference_mode():
+        cos, sin = torch.rand(5, 64), torch.rand(5, 64)
+        t1 = S._ROTARY_TABLES.get(cos, sin, 0)
+        assert S._ROTARY_TABLES.get(cos, sin, 0) is t1                    # within a pass: reused
+        cos.add_(1.0)                                                     # no version counter to notice this by
+        assert S._ROTARY_TABLES.get(cos, sin, 0) is t1
+        S._drop_rotary_tables(model, ())                                  # what the hook does when a pass starts
+        t2 = S._ROTARY_TABLES.get(cos, sin, 0)
+        assert t2 is not t1 and torch.equal(t2[:, :, 0], cos[:, 0::2].float())
+    S.swap_out(model)
+    assert "_tt_rotary_hook" not in model.__dict__ and len(model._forward_pre_hooks) == 0
+    assert not S._ROTARY_TABLES.entries
