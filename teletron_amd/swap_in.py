@@ -258,10 +258,17 @@ def _fused_rmsnorm_forward(self, x: torch.Tensor) -> torch.Tensor:
     return type(self).forward(self, x)
 
 
+def _aligned_or_copied(t: torch.Tensor) -> bool:
+    """What the op will hand to the kernel is 16-byte aligned: a fresh contiguous copy, or the tensor itself."""
+    return not t.is_contiguous() or t.data_ptr() % 16 == 0
+
+
 def _gate_fusable(x, gate, residual) -> bool:
+    # the gated residual add has no element-wise path: rows of a multiple of 8 elements, 16-byte aligned tensors
     return (isinstance(x, torch.Tensor) and isinstance(residual, torch.Tensor) and residual.dtype == torch.bfloat16
             and x.shape == residual.shape and residual.device == x.device and x.shape[-1] % 8 == 0
-            and modulation_fusable(x, gate))
+            and modulation_fusable(x, gate) and _aligned_or_copied(x) and _aligned_or_copied(residual)
+            and _aligned_or_copied(gate))
 
 
 def _fused_gate_forward(self, x, gate, residual):
