@@ -14,7 +14,7 @@ import pytest
 import torch
 
 from oracle import norm_oracle as O
-from test_gpu_parity import DEV, assert_bf16_close, rand_bf16
+from test_gpu_parity import DEV, WIDTHS, assert_bf16_close, rand_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -52,6 +52,32 @@ def test_adaln_reference_modules(rows, cols):
     # and it stays close to the gradient computed from x itself (x_norm carries one bf16 rounding)
     dxe, _, _ = O.adaln_backward(dy, x, scale, 1e-6, 1)
     torch.testing.assert_close(dinp.double().cpu(), dxe.reshape(rows, cols), rtol=2e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("rows", [3, 530])
+@pytest.mark.parametrize("cols", WIDTHS + [1001, 77])
+def test_adaln_forward_with_x_norm_every_kernel_variant(rows, cols):
+    """tt_launch_adaln_forward runs a kernel family of its own (the forward that also stores x_norm):
+    every wide and narrow variant, full and ragged, and the element-wise path, through the C ABI
+    against the oracle; 530 rows give every workgroup of a cache-resident launch several tiles."""
+    from teletron_amd import cabi
+    x = rand_bf16(rows, cols, seed=7 * rows + cols, offset=-0.2)
+    scale, shift = rand_bf16(cols, seed=5, scale=0.1), rand_bf16(cols, seed=6, scale=0.1)
+    xd, scd, shd = (t.to(DEV) for t in (x, scale, shift))
+    out = torch.full_like(xd, float("nan"))
+    x_norm = torch.full_like(xd, float("nan"))
+    invvar = torch.full((rows,), float("nan"), dtype=torch.float32, device=DEV)
+    cabi.call("tt_launch_adaln_forward", out.data_ptr(), x_norm.data_ptr(), xd.data_ptr(), scd.data_ptr(), shd.data_ptr(),
+              rows, cols, 1e-6, invvar.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    yo, xho, _, ro = O.adaln_forward(x, scale, shift, 1e-6, 1)
+    assert_bf16_close(out, yo, "output")
+    assert_bf16_close(x_norm, xho, "x_norm")
+    torch.testing.assert_close(invvar.double().cpu(), ro, rtol=1e-5, atol=0)
+    # the same output as the forward without x_norm, bit for bit (same arithmetic, other launch plan)
+    y2 = torch.empty_like(xd)
+    cabi.call("tt_adaln_forward", y2.data_ptr(), xd.data_ptr(), scd.data_ptr(), shd.data_ptr(), None, None,
+              rows, cols, rows, 1e-6, torch.cuda.current_stream().cuda_stream)
+    assert torch.equal(out, y2)
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 128), (4099, 128), (33, 1536), (257, 5120), (64, 72)])
